@@ -41,6 +41,8 @@ def find_architecture(cfg: Mapping[str, Any], arch: Optional[str] = None) -> Arc
                 return a
         raise ConfigError(f"unknown architecture {arch!r}; registered: {sorted(_REGISTRY)}")
     names = list(cfg.get("architectures") or [])
+    if isinstance(cfg.get("architecture"), str):           # (some families name one architecture, not a list)
+        names.append(cfg["architecture"])
     model_type = cfg.get("model_type")
     for a in _REGISTRY.values():
         if any(n == a.name for n in names) or (model_type is not None and model_type in a.aliases):

@@ -113,3 +113,9 @@ class ModelSpec:
     max_position: int
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
+    # The embedding: rows of the table times `embedding_scale`, plus a position vector over the model's width
+    # (`embedding_position`, kind "sinusoidal" with its `base`; None: none).  `reinject_before`: runs of the
+    # order (indices into `order`) right before which the embedding's output is added into the stream again.
+    embedding_scale: float = 1.0
+    embedding_position: Optional[PositionSpec] = None
+    reinject_before: Tuple[int, ...] = ()

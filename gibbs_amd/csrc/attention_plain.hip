@@ -5,7 +5,9 @@
 //   row n, head h (kv head g = h / (nh / nkv)), position p = pos[n], request r = row_req[n]:
 //   visible keys are lo .. p with lo = max(0, p - window + 1) (window 0: all keys);
 //   s_k = (q . K[k]) * scale (+ slopes[h] * (k - p) when the position encoding is a linear bias over
-//   the distance);  out = sum_k softmax(s)_k V[k], maxima and sums in float32.
+//   the distance; + bias[min(p - k, bias_len - 1)][h] when it is a table over the distance);
+//   out = sum_k softmax(s)_k V[k], maxima and sums in float32.  Values may have a head size of their
+//   own (vd): value pages are [page, kv head, slot in page, vd] and a row of out holds nh * vd.
 // Key k of request r lives in page table[r][k / ps] at slot k % ps; pages are
 // [page, kv head, slot in page, hd].  Visibility is by position only; what else a page holds is
 // never read.  One wave per (row, head).  Keys are taken in blocks of 64 aligned to absolute key
@@ -27,6 +29,9 @@ struct AttnArgs {
   float scale;
   int window;
   const float* slopes;  // [nh] or null: s_k += slopes[h] * (k - p)
+  int vd;               // head size of the values
+  const float* bias;    // [bias_len, nh] or null: s_k += bias[min(p - k, bias_len - 1)][h]
+  int bias_len;
 };
 
 template <typename T>
@@ -39,7 +44,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
   const int h_raw = blockIdx.y * 4 + wave;
   const bool active = h_raw < a.nh;
   const int h = active ? h_raw : a.nh - 1;
-  const int hd = a.hd;
+  const int hd = a.hd, vd = a.vd;
   const int g = h / (a.nh / a.nkv);
   const int p = a.pos[n];
   const int* table = a.table + (size_t)a.row_req[n] * a.max_pages;
@@ -53,10 +58,10 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
   float m = -INFINITY, l = 0.f;
   float acc[DPL] = {};
 
-  auto row_of = [&](const T* pages, int key) -> const T* {
+  auto row_of = [&](const T* pages, int key, int width) -> const T* {
     int page = table[key / a.page_size];
     page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
-    return pages + (((size_t)page * a.nkv + g) * a.page_size + key % a.page_size) * hd;
+    return pages + (((size_t)page * a.nkv + g) * a.page_size + key % a.page_size) * width;
   };
 
   for (int kb = lo / WAVE * WAVE; kb <= hi; kb += WAVE) {
@@ -64,11 +69,12 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
     const bool valid = key >= lo && key <= hi;
     float s = -INFINITY;
     if (valid) {
-      const T* kr = row_of(kpages, key);
+      const T* kr = row_of(kpages, key, hd);
       float dot = 0.f;
       for (int e = 0; e < hd; ++e) dot = fmaf(sq[wave][e], to_float(kr[e]), dot);
       s = dot * a.scale;
       if (a.slopes) s += a.slopes[h] * (float)(key - p);
+      if (a.bias) s += a.bias[(size_t)min(p - key, a.bias_len - 1) * a.nh + h];
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float w = valid ? expf(s - m_new) : 0.f;
@@ -79,36 +85,39 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
     const int k_end = min(WAVE, hi - kb + 1);
     for (int kk = max(0, lo - kb); kk < k_end; ++kk) {
       const float wk = __shfl(w, kk, WAVE);
-      const T* vr = row_of(vpages, kb + kk);
+      const T* vr = row_of(vpages, kb + kk, vd);
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         const int e = lane + i * WAVE;
-        if (e < hd) acc[i] = fmaf(wk, to_float(vr[e]), acc[i]);
+        if (e < vd) acc[i] = fmaf(wk, to_float(vr[e]), acc[i]);
       }
     }
     m = m_new;
   }
-  T* o = out + (size_t)n * a.ldo + (size_t)h * hd;
+  T* o = out + (size_t)n * a.ldo + (size_t)h * vd;
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
     const int e = lane + i * WAVE;
-    if (e < hd) o[e] = from_float<T>(acc[i] * inv);
+    if (e < vd) o[e] = from_float<T>(acc[i] * inv);
   }
 }
 }  // namespace
 
-GIBBS_EXPORT int gibbs_attention_plain(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
-                                       const int* pos, const int* row_req, const int* table, int max_pages,
-                                       int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                       long ldo, float scale, int window, const float* slopes, hipStream_t stream) {
-  GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
+// The general entry point: values of head size vd, and an optional table of score biases over the distance.
+GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                               const int* pos, const int* row_req, const int* table, int max_pages,
+                                               int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
+                                               long ldq, long ldo, float scale, int window, const float* slopes,
+                                               const float* bias, int bias_len, hipStream_t stream) {
+  GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "attention: bad sizes rows=%d heads=%d kv=%d hd=%d vd=%d", n_rows, nh, nkv, hd, vd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention: %d heads are not a multiple of %d kv heads", nh, nkv);
-  GIBBS_REQUIRE(hd <= MAX_HD, "attention: head size %d above %d", hd, MAX_HD);
-  GIBBS_REQUIRE(ldq >= (long)nh * hd && ldo >= (long)nh * hd, "attention: row strides shorter than heads * hd");
+  GIBBS_REQUIRE(hd <= MAX_HD && vd <= MAX_HD, "attention: head sizes %d, %d above %d", hd, vd, MAX_HD);
+  GIBBS_REQUIRE(ldq >= (long)nh * hd && ldo >= (long)nh * vd, "attention: row strides shorter than heads * head size");
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention: bad cache geometry");
+  GIBBS_REQUIRE(!bias || bias_len > 0, "attention: an empty table of score biases");
   if (n_rows == 0) return 0;
-  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes};
+  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes, vd, bias, bias_len};
   dim3 grid(n_rows, ceil_div(nh, 4));
   GIBBS_REQUIRE(grid.y <= 65535, "attention: too many heads (%d)", nh);
   if (dtype == GIBBS_F32)
@@ -118,4 +127,12 @@ GIBBS_EXPORT int gibbs_attention_plain(const void* q, const void* kpages, const 
   else
     return gibbs_fail("attention: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("attention");
+}
+
+GIBBS_EXPORT int gibbs_attention_plain(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                       const int* pos, const int* row_req, const int* table, int max_pages,
+                                       int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                       long ldo, float scale, int window, const float* slopes, hipStream_t stream) {
+  return gibbs_attention_plain_general(q, kpages, vpages, out, dtype, pos, row_req, table, max_pages, page_size, num_pages, n_rows,
+                                       nh, nkv, hd, hd, ldq, ldo, scale, window, slopes, nullptr, 0, stream);
 }

@@ -33,6 +33,30 @@ __global__ void glu_bf16x8_kernel(const bf16* __restrict__ gu, bf16* __restrict_
   *(uint4*)(out + (size_t)n * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
+// The clamped variant:  g = min(gate, limit), u = clamp(up, -limit, limit);  out = g * sigmoid(alpha * g) * (u + 1).
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float alpha, float limit) {
+  const int n = blockIdx.x;
+  const int f = blockIdx.y * blockDim.x + threadIdx.x;
+  if (f >= F) return;
+  const float g = fminf(to_float(gu[(size_t)n * 2 * F + f]), limit);
+  const float u = fminf(fmaxf(to_float(gu[(size_t)n * 2 * F + F + f]), -limit), limit);
+  out[(size_t)n * F + f] = from_float<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+}
+
+GIBBS_EXPORT int gibbs_glu_clamped(const void* gu, void* out, int dtype, int n, int F, float alpha, float limit, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && F > 0 && F <= 65535 * 256, "glu: bad sizes n=%d F=%d", n, F);
+  if (n == 0) return 0;
+  dim3 grid(n, ceil_div(F, 256));
+  if (dtype == GIBBS_F32)
+    glu_clamped_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, F, alpha, limit);
+  else if (dtype == GIBBS_BF16)
+    glu_clamped_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, F, alpha, limit);
+  else
+    return gibbs_fail("glu: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("glu");
+}
+
 GIBBS_EXPORT int gibbs_glu(const void* gu, void* out, int dtype, int n, int F, int act, hipStream_t stream) {
   GIBBS_REQUIRE(n >= 0 && F > 0, "glu: bad sizes n=%d F=%d", n, F);
   GIBBS_REQUIRE(act >= 0 && act < ACT_COUNT, "glu: unknown activation %d", act);

@@ -1,0 +1,391 @@
+// Kernels of mixers that carry a matrix state from token to token: the gated delta rule and the
+// decayed outer-product rule of RWKV-style time mixing, with what surrounds them (short causal
+// convolutions with state, unit vectors, decays, the shift by one token, the gated norm of a head's
+// read-out).  Everything that enters a recurrence is float32, and so is the state.
+//
+// A step's rows are a ragged batch: request r brings rows cu[r] .. cu[r+1]-1 and keeps its state in
+// slot[r] of the arena.  Every kernel treats a token the same way wherever its step was cut: the
+// recurrences walk a request's rows in order with a fixed order of additions per token, so a prompt
+// in one step, in portions or token by token gives the same bits.
+#include "common.h"
+
+namespace {
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float activate_gate(float z, int act) {   // 0: silu, 1: sigmoid
+  return act == 1 ? sigmoid_f(z) : z * sigmoid_f(z);
+}
+
+// ------------------------------------------------------------------------------------------------ short causal convolution
+// y[n, c] = silu(sum_j taps[c, j] * x[t - (K-1) + j, c]): the last tap is the current token's; inputs before the
+// step's first row come from the request's state (its last K-1 inputs, oldest first; zeros at a sequence's start).
+template <typename T>
+__global__ void causal_conv_silu_kernel(const T* __restrict__ in, long ld, const float* __restrict__ taps,
+                                        const float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
+                                        const int* __restrict__ cu, const int* __restrict__ slot, float* __restrict__ out,
+                                        int C, int K) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int r = row_req[n], first = cu[r], t = n - first;
+  const float* st = state + (size_t)slot[r] * slot_stride;
+  float acc = 0.f;
+  for (int j = 0; j < K; ++j) {
+    const int tt = t - (K - 1) + j;
+    const float xv = tt >= 0 ? to_float(in[(size_t)(first + tt) * ld + c]) : st[(size_t)(K - 1 + tt) * C + c];
+    acc = fmaf(taps[(size_t)c * K + j], xv, acc);
+  }
+  out[(size_t)n * C + c] = acc * sigmoid_f(acc);
+}
+
+// The state after the step: the last K-1 inputs of the request (what the step brought, and before that what
+// the state held).  One thread per (request, channel), entries in ascending order: entry i reads entry
+// i + rows of the old state, which has not been written yet.
+template <typename T>
+__global__ void causal_conv_state_kernel(const T* __restrict__ in, long ld, float* __restrict__ state, long slot_stride,
+                                         const int* __restrict__ cu, const int* __restrict__ slot, int C, int K) {
+  const int r = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int first = cu[r], rows = cu[r + 1] - first;
+  float* st = state + (size_t)slot[r] * slot_stride;
+  for (int i = 0; i < K - 1; ++i) {
+    const int src = i + rows - (K - 1);
+    st[(size_t)i * C + c] = src >= 0 ? to_float(in[(size_t)(first + src) * ld + c]) : st[(size_t)(i + rows) * C + c];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ what the delta rule reads
+struct DeltaPrepArgs {
+  float* q;            // [N, G*D] float32, in place: unit vector * q_scale
+  float* k;            // [N, G*D] in place: unit vector
+  long ldqk;
+  const void* beta_raw;   // [N, ld_raw] in the activation type: W_b h
+  long ld_raw;
+  const void* a_head;     // head decay: [N, ld_raw] activation type, one per head (null with a_channel)
+  const float* a_channel; // channel decay: [N, H*D] float32
+  const float* dt_bias;   // [H] or [H*D]
+  const float* a_log;     // [H]
+  float* beta;            // [N, H]
+  float* decay;           // [N, H] or [N, H*D]
+  int G, H, D;
+  float q_scale, unit_eps;
+};
+
+// Block y < G: q and k of kv head y become unit vectors x / sqrt(sum x^2 + eps) (q times q_scale).  Block
+// y >= G: head y - G's beta = sigmoid(.) and decay g = exp(-exp(A_log) * softplus(a + dt_bias)).
+template <typename T>
+__global__ __launch_bounds__(64) void delta_prep_kernel(DeltaPrepArgs a) {
+  const int n = blockIdx.x, lane = threadIdx.x;
+  if ((int)blockIdx.y < a.G) {
+    const int g = blockIdx.y;
+    float* q = a.q + (size_t)n * a.ldqk + (size_t)g * a.D;
+    float* k = a.k + (size_t)n * a.ldqk + (size_t)g * a.D;
+    float sq = 0.f, sk = 0.f;
+    for (int i = lane; i < a.D; i += WAVE) {
+      sq = fmaf(q[i], q[i], sq);
+      sk = fmaf(k[i], k[i], sk);
+    }
+    const float rq = a.q_scale / sqrtf(wave_sum(sq) + a.unit_eps), rk = 1.0f / sqrtf(wave_sum(sk) + a.unit_eps);
+    for (int i = lane; i < a.D; i += WAVE) {
+      q[i] *= rq;
+      k[i] *= rk;
+    }
+    return;
+  }
+  const int h = blockIdx.y - a.G;
+  const float rate = expf(a.a_log[h]);
+  if (lane == 0) a.beta[(size_t)n * a.H + h] = sigmoid_f(to_float(((const T*)a.beta_raw)[(size_t)n * a.ld_raw + h]));
+  if (a.a_channel) {
+    for (int i = lane; i < a.D; i += WAVE) {
+      const size_t at = (size_t)n * a.H * a.D + (size_t)h * a.D + i;
+      a.decay[at] = expf(-rate * softplus_f(a.a_channel[at] + a.dt_bias[h * a.D + i]));
+    }
+  } else if (lane == 0) {
+    const float z = to_float(((const T*)a.a_head)[(size_t)n * a.ld_raw + h]) + a.dt_bias[h];
+    a.decay[(size_t)n * a.H + h] = expf(-rate * softplus_f(z));
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ the recurrences
+enum { RULE_DELTA = 0, RULE_OUTER = 1 };
+struct RecurrenceArgs {
+  const void* q;       // delta: unit q * scale; outer: the receptance r.  [N, G*D]
+  const void* k;       // [N, G*D]
+  const void* v;       // [N, H*V]
+  long ldq, ldk, ldv;
+  const float* decay;  // delta: g [N, H] (per_channel 0) or [N, H*D]; outer: w [N, H*D]
+  int per_channel;
+  const float* beta;   // delta: [N, H]
+  const float* bonus;  // outer: u [H, D], for the current token only
+  float* state;        // [slots][H][D][V] float32
+  long slot_stride;
+  const int* cu;
+  const int* slot;
+  float* out;          // [N, H*V] float32
+  int H, G, D, V;
+};
+
+// One wave per (request, head, 16 columns of the state).  A column of S [D, V] is spread over 4 lanes (key
+// channel i belongs to lane part i % 4, so a lane holds DPT = ceil(D / 4) values in registers); sums over the
+// key channels are folded over those 4 lanes.  The operands of 8 tokens at a time go through LDS.
+//   delta:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   outer:  o = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T
+template <typename TIn, int RULE, int DPT>
+__global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
+  constexpr int PARTS = 4, COLS = 16, TOK = 8, DMAX = DPT * PARTS;
+  __shared__ float sq[TOK][DMAX], sk[TOK][DMAX], sd[TOK][DMAX], sv[TOK][COLS], sb[TOK], sg[TOK];
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int col = lane / PARTS, part = lane % PARTS;
+  const int j = blockIdx.z * COLS + col;
+  const int kvh = h / (a.H / a.G);
+  const int first = a.cu[r], rows = a.cu[r + 1] - first;
+  const int D = a.D, V = a.V;
+  float* st = a.state + (size_t)a.slot[r] * a.slot_stride + (size_t)h * D * V;
+  float S[DPT], bonus[DPT];
+#pragma unroll
+  for (int ii = 0; ii < DPT; ++ii) {
+    const int i = ii * PARTS + part;
+    S[ii] = (i < D && j < V) ? st[(size_t)i * V + j] : 0.f;
+    bonus[ii] = (RULE == RULE_OUTER && i < D) ? a.bonus[(size_t)h * D + i] : 0.f;
+  }
+  const TIn* q = (const TIn*)a.q;
+  const TIn* k = (const TIn*)a.k;
+  const TIn* v = (const TIn*)a.v;
+  const bool channel_decay = RULE == RULE_OUTER || a.per_channel;
+  for (int t0 = 0; t0 < rows; t0 += TOK) {
+    const int nt = min(TOK, rows - t0);
+    __syncthreads();
+    for (int idx = lane; idx < TOK * DMAX; idx += WAVE) {
+      const int t = idx / DMAX, i = idx % DMAX;
+      const bool live = t < nt && i < D;
+      const size_t row = (size_t)(first + t0 + (t < nt ? t : 0));
+      sq[t][i] = live ? to_float(q[row * a.ldq + (size_t)kvh * D + i]) : 0.f;
+      sk[t][i] = live ? to_float(k[row * a.ldk + (size_t)kvh * D + i]) : 0.f;
+      if (channel_decay) sd[t][i] = live ? a.decay[row * a.H * D + (size_t)h * D + i] : 1.f;
+    }
+    for (int idx = lane; idx < TOK * COLS; idx += WAVE) {
+      const int t = idx / COLS, c = idx % COLS, jj = blockIdx.z * COLS + c;
+      sv[t][c] = (t < nt && jj < V) ? to_float(v[(size_t)(first + t0 + t) * a.ldv + (size_t)h * V + jj]) : 0.f;
+    }
+    if (RULE == RULE_DELTA && lane < TOK) {
+      const bool live = lane < nt;
+      const size_t row = (size_t)(first + t0 + (live ? lane : 0));
+      sb[lane] = live ? a.beta[row * a.H + h] : 0.f;
+      sg[lane] = (live && !a.per_channel) ? a.decay[row * a.H + h] : 1.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+      const float vj = sv[t][col];
+      float o = 0.f;
+      if (RULE == RULE_DELTA) {
+        const float g_head = sg[t];
+        float dot = 0.f;
+#pragma unroll
+        for (int ii = 0; ii < DPT; ++ii) {
+          const int i = ii * PARTS + part;
+          const float s = S[ii] * (channel_decay ? sd[t][i] : g_head);
+          S[ii] = s;
+          dot = fmaf(s, sk[t][i], dot);
+        }
+        dot += __shfl_xor(dot, 1, WAVE);
+        dot += __shfl_xor(dot, 2, WAVE);
+        const float u = sb[t] * (vj - dot);
+#pragma unroll
+        for (int ii = 0; ii < DPT; ++ii) {
+          const int i = ii * PARTS + part;
+          const float s = fmaf(sk[t][i], u, S[ii]);
+          S[ii] = s;
+          o = fmaf(s, sq[t][i], o);
+        }
+      } else {
+#pragma unroll
+        for (int ii = 0; ii < DPT; ++ii) {
+          const int i = ii * PARTS + part;
+          const float kv = sk[t][i] * vj;
+          o = fmaf(sq[t][i], fmaf(bonus[ii], kv, S[ii]), o);
+          S[ii] = fmaf(sd[t][i], S[ii], kv);
+        }
+      }
+      o += __shfl_xor(o, 1, WAVE);
+      o += __shfl_xor(o, 2, WAVE);
+      if (part == 0 && j < V) a.out[(size_t)(first + t0 + t) * a.H * V + (size_t)h * V + j] = o;
+    }
+  }
+#pragma unroll
+  for (int ii = 0; ii < DPT; ++ii) {
+    const int i = ii * PARTS + part;
+    if (i < D && j < V) st[(size_t)i * V + j] = S[ii];
+  }
+}
+
+template <typename TIn, int RULE>
+int launch_recurrence(const RecurrenceArgs& a, int n_req, hipStream_t stream) {
+  const dim3 grid(n_req, a.H, ceil_div(a.V, 16));
+  if (a.D <= 32) recurrence_kernel<TIn, RULE, 8><<<grid, 64, 0, stream>>>(a);
+  else if (a.D <= 64) recurrence_kernel<TIn, RULE, 16><<<grid, 64, 0, stream>>>(a);
+  else if (a.D <= 128) recurrence_kernel<TIn, RULE, 32><<<grid, 64, 0, stream>>>(a);
+  else recurrence_kernel<TIn, RULE, 64><<<grid, 64, 0, stream>>>(a);
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ a head's read-out, normed and gated
+// y[n, h, :] = o[n, h, :] / sqrt(mean(o^2) + eps) * gain[(h V + j) % gain_len] * act(gate[n, h V + j])
+template <typename T>
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ gain,
+                                                            int gain_len, const T* __restrict__ gate, long ld_gate,
+                                                            T* __restrict__ y, int H, int V, float eps, int act) {
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* row = o + (size_t)n * H * V + (size_t)h * V;
+  float ss = 0.f;
+  for (int j = lane; j < V; j += WAVE) ss = fmaf(row[j], row[j], ss);
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
+  for (int j = lane; j < V; j += WAVE) {
+    const int c = h * V + j;
+    const float g = activate_gate(to_float(gate[(size_t)n * ld_gate + c]), act);
+    y[(size_t)n * H * V + c] = from_float<T>(row[j] * inv * gain[c % gain_len] * g);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ shift by one token
+// out[s, n, c] = h[n, c] + (prev[n, c] - h[n, c]) * mu[s, c]; prev is the request's previous token's h: the row
+// before, or for a step's first row the request's state (zeros at a sequence's start).
+template <typename T>
+__global__ void token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int n_mix,
+                                   const float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
+                                   const int* __restrict__ cu, const int* __restrict__ slot, T* __restrict__ out, int N, int W) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int r = row_req[n];
+  const float cur = to_float(h[(size_t)n * W + c]);
+  const float prev = n > cu[r] ? to_float(h[(size_t)(n - 1) * W + c]) : state[(size_t)slot[r] * slot_stride + c];
+  for (int s = 0; s < n_mix; ++s)
+    out[((size_t)s * N + n) * W + c] = from_float<T>(fmaf(prev - cur, mu[(size_t)s * W + c], cur));
+}
+template <typename T>
+__global__ void token_shift_state_kernel(const T* __restrict__ h, float* __restrict__ state, long slot_stride,
+                                         const int* __restrict__ cu, const int* __restrict__ slot, int W) {
+  const int r = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  state[(size_t)slot[r] * slot_stride + c] = to_float(h[(size_t)(cu[r + 1] - 1) * W + c]);
+}
+
+// out = tanh(in) (float32 in, the activation type out); and w = exp(-exp(z + w0)) in place.
+template <typename T>
+__global__ void tanh_kernel(const float* __restrict__ in, T* __restrict__ out, long count) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) out[i] = from_float<T>(tanhf(in[i]));
+}
+__global__ void double_exp_decay_kernel(float* __restrict__ z, const float* __restrict__ bias, long count, int C) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) z[i] = expf(-expf(z[i] + bias[i % C]));
+}
+}  // namespace
+
+#define BY_DTYPE(dtype, what, call_f32, call_bf16)         \
+  do {                                                     \
+    if ((dtype) == GIBBS_F32) { call_f32; }                \
+    else if ((dtype) == GIBBS_BF16) { call_bf16; }         \
+    else return gibbs_fail(what ": unknown dtype %d", (dtype)); \
+  } while (0)
+
+GIBBS_EXPORT int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
+                                        const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req,
+                                        int C, int K, int update_state, hipStream_t stream) {
+  GIBBS_REQUIRE(in && taps && state && out && n_rows > 0 && n_req > 0 && C > 0 && K >= 1 && ld >= C && slot_stride >= (long)(K - 1) * C,
+                "causal_conv: bad operands rows=%d requests=%d C=%d K=%d", n_rows, n_req, C, K);
+  const dim3 rows(n_rows, ceil_div(C, 256)), reqs(n_req, ceil_div(C, 256));
+  BY_DTYPE(dtype, "causal_conv",
+           (causal_conv_silu_kernel<float><<<rows, 256, 0, stream>>>((const float*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K)),
+           (causal_conv_silu_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K)));
+  if (update_state && K > 1)
+    BY_DTYPE(dtype, "causal_conv",
+             (causal_conv_state_kernel<float><<<reqs, 256, 0, stream>>>((const float*)in, ld, state, slot_stride, cu, slot, C, K)),
+             (causal_conv_state_kernel<bf16><<<reqs, 256, 0, stream>>>((const bf16*)in, ld, state, slot_stride, cu, slot, C, K)));
+  GIBBS_LAUNCH_STATUS("causal_conv");
+}
+
+GIBBS_EXPORT int gibbs_delta_prep(float* q, float* k, long ldqk, const void* beta_raw, const void* a_head, long ld_raw, int dtype,
+                                  const float* a_channel, const float* dt_bias, const float* a_log, float* beta, float* decay,
+                                  int n_rows, int G, int H, int D, float q_scale, float unit_eps, hipStream_t stream) {
+  GIBBS_REQUIRE(q && k && beta_raw && (a_head || a_channel) && dt_bias && a_log && beta && decay && n_rows > 0 && G > 0 && H > 0 && D > 0,
+                "delta_prep: bad operands rows=%d kv heads=%d heads=%d D=%d", n_rows, G, H, D);
+  DeltaPrepArgs a{q, k, ldqk, beta_raw, ld_raw, a_channel ? nullptr : a_head, a_channel, dt_bias, a_log, beta, decay, G, H, D, q_scale, unit_eps};
+  const dim3 grid(n_rows, G + H);
+  BY_DTYPE(dtype, "delta_prep", (delta_prep_kernel<float><<<grid, 64, 0, stream>>>(a)), (delta_prep_kernel<bf16><<<grid, 64, 0, stream>>>(a)));
+  GIBBS_LAUNCH_STATUS("delta_prep");
+}
+
+namespace {
+int check_recurrence(const char* what, int n_req, int H, int G, int D, int V, long slot_stride) {
+  GIBBS_REQUIRE(n_req > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && V > 0,
+                "%s: bad sizes requests=%d heads=%d kv heads=%d D=%d (up to 256) V=%d", what, n_req, H, G, D, V);
+  GIBBS_REQUIRE(slot_stride >= (long)H * D * V, "%s: a slot of %ld floats cannot hold %d x %d x %d", what, slot_stride, H, D, V);
+  return 0;
+}
+}  // namespace
+
+// The gated delta rule over a ragged batch; q, k (unit vectors, q scaled), v, beta, decay float32.
+GIBBS_EXPORT int gibbs_delta_rule(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* beta, const float* decay,
+                                  int per_channel, float* state, long slot_stride, const int* cu, const int* slot, float* out,
+                                  int n_req, int H, int G, int D, int V, hipStream_t stream) {
+  GIBBS_REQUIRE(q && k && v && beta && decay && state && cu && slot && out && ldqk >= (long)G * D && ldv >= (long)H * V, "delta_rule: null operand or short rows");
+  if (check_recurrence("delta_rule", n_req, H, G, D, V, slot_stride)) return 1;
+  RecurrenceArgs a{q, k, v, ldqk, ldqk, ldv, decay, per_channel, beta, nullptr, state, slot_stride, cu, slot, out, H, G, D, V};
+  launch_recurrence<float, RULE_DELTA>(a, n_req, stream);
+  GIBBS_LAUNCH_STATUS("delta_rule");
+}
+
+// o_t = (S + diag(bonus) k v^T)^T r; S <- diag(w) S + k v^T; r, k, v [N, H*D] in the activation type, w float32.
+GIBBS_EXPORT int gibbs_decayed_outer_rule(const void* r, const void* k, const void* v, int dtype, const float* w, const float* bonus,
+                                          float* state, long slot_stride, const int* cu, const int* slot, float* out, int n_req,
+                                          int H, int D, hipStream_t stream) {
+  GIBBS_REQUIRE(r && k && v && w && bonus && state && cu && slot && out, "decayed_outer_rule: null operand");
+  if (check_recurrence("decayed_outer_rule", n_req, H, H, D, D, slot_stride)) return 1;
+  RecurrenceArgs a{r, k, v, (long)H * D, (long)H * D, (long)H * D, w, 1, nullptr, bonus, state, slot_stride, cu, slot, out, H, H, D, D};
+  BY_DTYPE(dtype, "decayed_outer_rule", (launch_recurrence<float, RULE_OUTER>(a, n_req, stream)),
+           (launch_recurrence<bf16, RULE_OUTER>(a, n_req, stream)));
+  GIBBS_LAUNCH_STATUS("decayed_outer_rule");
+}
+
+GIBBS_EXPORT int gibbs_head_norm_gate(const float* o, const float* gain, int gain_len, const void* gate, long ld_gate, void* y,
+                                      int dtype, int n_rows, int H, int V, float eps, int act, hipStream_t stream) {
+  GIBBS_REQUIRE(o && gain && gate && y && n_rows > 0 && H > 0 && V > 0 && gain_len > 0 && ld_gate >= (long)H * V && (act == 0 || act == 1),
+                "head_norm_gate: bad operands rows=%d heads=%d V=%d", n_rows, H, V);
+  const dim3 grid(n_rows, H);
+  BY_DTYPE(dtype, "head_norm_gate",
+           (head_norm_gate_kernel<float><<<grid, 64, 0, stream>>>(o, gain, gain_len, (const float*)gate, ld_gate, (float*)y, H, V, eps, act)),
+           (head_norm_gate_kernel<bf16><<<grid, 64, 0, stream>>>(o, gain, gain_len, (const bf16*)gate, ld_gate, (bf16*)y, H, V, eps, act)));
+  GIBBS_LAUNCH_STATUS("head_norm_gate");
+}
+
+GIBBS_EXPORT int gibbs_token_shift(const void* h, int dtype, const float* mu, int n_mix, float* state, long slot_stride,
+                                   const int* row_req, const int* cu, const int* slot, void* out, int n_rows, int n_req, int W,
+                                   int update_state, hipStream_t stream) {
+  GIBBS_REQUIRE(h && mu && state && out && n_rows > 0 && n_req > 0 && W > 0 && n_mix > 0 && slot_stride >= W,
+                "token_shift: bad operands rows=%d requests=%d W=%d", n_rows, n_req, W);
+  const dim3 rows(n_rows, ceil_div(W, 256)), reqs(n_req, ceil_div(W, 256));
+  BY_DTYPE(dtype, "token_shift",
+           (token_shift_kernel<float><<<rows, 256, 0, stream>>>((const float*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (float*)out, n_rows, W)),
+           (token_shift_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (bf16*)out, n_rows, W)));
+  if (update_state)
+    BY_DTYPE(dtype, "token_shift",
+             (token_shift_state_kernel<float><<<reqs, 256, 0, stream>>>((const float*)h, state, slot_stride, cu, slot, W)),
+             (token_shift_state_kernel<bf16><<<reqs, 256, 0, stream>>>((const bf16*)h, state, slot_stride, cu, slot, W)));
+  GIBBS_LAUNCH_STATUS("token_shift");
+}
+
+GIBBS_EXPORT int gibbs_tanh_rows(const float* in, void* out, int dtype, long count, hipStream_t stream) {
+  GIBBS_REQUIRE(in && out && count > 0, "tanh: bad operands");
+  BY_DTYPE(dtype, "tanh", (tanh_kernel<float><<<ceil_div(count, 256), 256, 0, stream>>>(in, (float*)out, count)),
+           (tanh_kernel<bf16><<<ceil_div(count, 256), 256, 0, stream>>>(in, (bf16*)out, count)));
+  GIBBS_LAUNCH_STATUS("tanh");
+}
+
+GIBBS_EXPORT int gibbs_double_exp_decay(float* z, const float* bias, long count, int C, hipStream_t stream) {
+  GIBBS_REQUIRE(z && bias && count > 0 && C > 0, "double_exp_decay: bad operands");
+  double_exp_decay_kernel<<<ceil_div(count, 256), 256, 0, stream>>>(z, bias, count, C);
+  GIBBS_LAUNCH_STATUS("double_exp_decay");
+}

@@ -46,6 +46,7 @@ long ceil_div_l(long a, long b) { return (a + b - 1) / b; }
 constexpr int FUSED_ROWS = 64;            // rows that the few-row products (and so the fused decode kernels) take
 constexpr int SKINNY_ROWS = 64;           // rows up to which a plain product takes the weight-streaming kernel
 constexpr int SKINNY_ROWS_F32_OUT = 48;   // the same for float32 output (the head: it streams faster than the tiled product)
+constexpr int ACT_CLAMPED = 4;            // the gated feed-forward's clamped activation (beside activation.h's codes 0 .. 3)
 constexpr int MATRIX_SLICE_PAGES = 510;   // page ids of a key slice that the decode attention's matrix-core walk keeps in LDS
 
 // Ranges of k that the few-row product is cut into so that at least `want_blocks` workgroups run (a
@@ -116,7 +117,7 @@ LinearChoice choose_linear(bool bf16_run, int n, int O, int I, bool aligned, boo
   if (!bf16_run) return {LIN_F32, 1};                    // the true 32-bit product, plain FMA in ascending k
   if (!aligned) return {LIN_PLAIN, 1};                   // what the matrix-core kernels refuse
   if (n <= (out_f32 && !partial_ok ? SKINNY_ROWS_F32_OUT : SKINNY_ROWS)) return {LIN_SKINNY, partial_ok ? skinny_splits(O, I) : 1};
-  if (!own_gemm && !out_f32) return {LIN_LIBRARY, 1};    // (the library writes bfloat16 only)
+  if (!own_gemm && !out_f32 && O % 8 == 0) return {LIN_LIBRARY, 1};    // (the library writes bfloat16 only, in rows of whole 16 bytes)
   return {LIN_TILED, 1};
 }
 bool aligned_for_matrix_cores(const void* x, long ldx, const void* w, int I) {
@@ -236,7 +237,7 @@ struct Exec {
   // y = x @ W^T in the precision of the run.  `out_f32`: float32 output; `partial_ok`: the caller takes
   // float32 partial sums; `use_packed`: the few-row kernel may read the tile-ordered copy.  Returns the
   // buffer ([N, O], or [parts, N, O] float32 with *parts >= 2).
-  void* linear(const void* x, const Matrix& m, int n, bool out_f32, bool partial_ok, bool use_packed, int* parts);
+  void* linear(const void* x, const Matrix& m, int n, bool out_f32, bool partial_ok, bool use_packed, int* parts, long ldx = 0);
   void linear_into(const void* x, const Matrix& m, int n, bool out_f32, bool use_packed, void* y);
   // adds what is pending and makes sure the bfloat16 mirror of x exists
   void with_mirror(float* x, Pending& pending, void** mirror);
@@ -259,6 +260,8 @@ struct NormPart {
   virtual void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const = 0;
   // an RMS norm whose gain is folded into the matrices that follow: the fused kernels do the rest of it
   virtual bool folded_rms(float* eps) const { return false; }
+  // the norm of a part's result before it is added (the stream is not touched); gives the delta's buffer back
+  virtual Pending run_on(Exec& e, Pending delta) const;
 };
 
 struct Body {
@@ -276,13 +279,17 @@ struct Plan {
   int hidden = 0, vocab = 0;
   const void* table = nullptr;
   int table_dtype = GIBBS_BF16;
+  float embed_scale = 1.0f;            // the table's rows are multiplied by it
+  const float* embed_inv_freq = nullptr;   // [hidden / 2]: a sinusoidal position vector is added to the rows
+  bool plain_embedding() const { return embed_scale == 1.0f && !embed_inv_freq && !reinjects; }
+  bool reinjects = false;              // the program adds the embedding's output into the stream again
   Matrix head;
   int tail = -1;            // the norm in front of the head
   int fused_rows = FUSED_ROWS;   // steps of at most this many decoded tokens take the fused decode kernels
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
   std::vector<std::unique_ptr<NormPart>> norms;
   std::vector<std::unique_ptr<Body>> bodies;
-  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP };
+  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT };
   struct Op {
     int kind, norm, body, value;   // value: what a body reads, an add adds, a drop drops
     int result;                    // the value that a norm or a body makes
@@ -302,11 +309,12 @@ Exec::Exec(const Plan& plan, const GibbsStepArgs& args)
   fused_step = few_rows && a.max_q == 1;
 }
 
-void* Exec::linear(const void* x, const Matrix& m, int n, bool out_f32, bool partial_ok, bool use_packed, int* parts) {
-  const LinearChoice c = choose_linear(bf16_run, n, m.O, m.I, aligned_for_matrix_cores(x, m.I, m.w, m.I), out_f32, partial_ok, p.own_gemm);
+void* Exec::linear(const void* x, const Matrix& m, int n, bool out_f32, bool partial_ok, bool use_packed, int* parts, long ldx) {
+  if (ldx == 0) ldx = m.I;     // (x may be a slice of wider rows)
+  const LinearChoice c = choose_linear(bf16_run, n, m.O, m.I, aligned_for_matrix_cores(x, ldx, m.w, m.I), out_f32, partial_ok, p.own_gemm);
   const long elem = !bf16_run || out_f32 || c.splits > 1 ? 4 : 2;
   void* y = take((long)c.splits * n * m.O * elem);
-  RUN(*this, run_linear(c, x, m.I, m, use_packed, y, n, out_f32, a.stream));
+  RUN(*this, run_linear(c, x, ldx, m, use_packed, y, n, out_f32, a.stream));
   if (parts) *parts = c.splits;
   return y;
 }
@@ -339,6 +347,10 @@ void Exec::skinny_residual(const void* y, const Matrix& m, float* x, void* mirro
 }
 
 // ---- norms
+Pending NormPart::run_on(Exec& e, Pending delta) const {
+  if (!e.status) e.status = gibbs_fail("step: this norm cannot be applied to a part's result");
+  return delta;
+}
 struct RmsNorm : NormPart {
   const float* gain = nullptr;   // null: folded into the matrices that follow
   float eps = 0.f;
@@ -357,6 +369,13 @@ struct RmsNorm : NormPart {
   bool folded_rms(float* e) const override {
     *e = eps;
     return gain == nullptr;
+  }
+  Pending run_on(Exec& e, Pending delta) const override {
+    const int N = e.a.n_rows, H = e.p.hidden;
+    Pending out{e.take((long)N * H * e.esize), 1};
+    RUN(e, gibbs_rmsnorm_rows(delta.data, std::max(delta.parts, 1), (long)N * H, gain, eps, out.data, e.p.dtype, N, H, e.a.stream));
+    e.give(delta.data);
+    return out;
   }
 };
 struct HostNorm : NormPart {
@@ -426,8 +445,16 @@ struct AttnBody : Body {
   const float* slopes = nullptr;      // a bias on the scores by distance: the plain kernel takes it
   GibbsHostRows hook = nullptr;       // something else done to q and k rows before k is cached
   void* hook_user = nullptr;
+  // what gibbs_plan_attention_extras sets: values of a head size of their own, q and k divided by their root mean
+  // square without a gain, a temperature on q that grows with the position, a table of score biases over the distance
+  int vd = 0;
+  int unit_qk = 0, temp_every = 0;
+  float temp_coef = 0.f;
+  const float* bias = nullptr;
+  int bias_len = 0;
+  bool extras() const { return vd != hd || unit_qk || temp_every > 0 || bias; }
   int cache_group() const override { return group; }
-  bool fast() const { return !slopes && !hook; }   // the fast kernels know rotations only (or no encoding at all)
+  bool fast() const { return !slopes && !hook && !extras(); }   // the fast kernels know rotations only (or no encoding at all)
   // what the kernel that takes the raw projection (q/k norm, rotation, cache write and attention in one) needs
   bool raw_ok() const { return fast() && owns && hd % 16 == 0 && hd <= 256 && (!inv_freq || rot % 16 == 0); }
   bool fusable(bool single) const override { return single && raw_ok() && qkv.I % 8 == 0 && (nh * hd) % 8 == 0; }
@@ -468,6 +495,11 @@ struct AttnBody : Body {
     const int N = e.a.n_rows, kv = owns ? nkv : 0;
     const int* table = e.table(group);
     const int width = e.width(group);
+    if (extras()) {
+      RUN(e, gibbs_qk_unit_kv(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, e.a.pos, e.a.row_req, table, width,
+                              page_size, num_pages, N, nh, kv, hd, vd, qk_eps, unit_qk, temp_coef, temp_every, e.a.stream));
+      return;
+    }
     if (!hook) {
       RUN(e, gibbs_qk_rope_kv(raw, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, q_gain, k_gain, qk_eps, inv_freq, rot,
                               variant, cos_sin, cos_sin && inv_freq ? table_len : 0, e.a.pos, e.a.row_req, owns ? table : nullptr,
@@ -492,7 +524,7 @@ struct AttnBody : Body {
   void* attend(Exec& e, void* raw) const {
     const GibbsStepArgs& a = e.a;
     const int N = a.n_rows, kv = owns ? nkv : 0;
-    const long ldq = (long)(nh + 2 * kv) * hd, ldo = (long)nh * hd;
+    const long ldq = (long)(nh + kv) * hd + (long)kv * vd, ldo = (long)nh * vd;
     void* att;
     if (e.bf16_run && a.max_q == 1 && raw_ok()) {
       att = attend_decoded(e, raw);
@@ -501,7 +533,7 @@ struct AttnBody : Body {
       const int* table = e.table(group);
       const int width = e.width(group);
       att = e.take((long)N * ldo * e.esize);
-      const bool fast_bf16 = e.bf16_run && !slopes;   // (the fast kernels take no score bias)
+      const bool fast_bf16 = e.bf16_run && !slopes && !extras();   // (the fast kernels take no score bias)
       if (fast_bf16 && a.max_q > 1 && hd % 16 == 0 && hd <= 128) {
         // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
         // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
@@ -518,8 +550,8 @@ struct AttnBody : Body {
       } else if (fast_bf16 && a.max_q == 1 && hd % 8 == 0) {
         decode_attention(e, raw, ldq, N, a.pos, a.row_req, att);
       } else {
-        RUN(e, gibbs_attention_plain(raw, kpages, vpages, att, e.p.dtype, a.pos, a.row_req, table, width, page_size, num_pages, N, nh,
-                                     nkv, hd, ldq, ldo, scale, window, slopes, a.stream));
+        RUN(e, gibbs_attention_plain_general(raw, kpages, vpages, att, e.p.dtype, a.pos, a.row_req, table, width, page_size, num_pages,
+                                             N, nh, nkv, hd, vd, ldq, ldo, scale, window, slopes, bias, bias_len, a.stream));
       }
     }
     return att;
@@ -541,7 +573,9 @@ struct GluBody : Body {
   Matrix gate_up, down;
   const void* gate_up_packed2 = nullptr;   // gate and up packed as two row groups, for the fused kernel
   int F = 0, act = 0;
-  bool fusable(bool) const override { return gate_up.I % 8 == 0 && F % 8 == 0; }   // (rows one by one: any few rows)
+  // act ACT_CLAMPED: min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1); the stand-alone kernel only
+  float alpha = 0.f, limit = 0.f;
+  bool fusable(bool) const override { return act != ACT_CLAMPED && gate_up.I % 8 == 0 && F % 8 == 0; }   // (rows one by one: any few rows)
   void fused(Exec& e, float eps, float* x, void* mirror) const override {
     const int N = e.a.n_rows, H = gate_up.I;
     void* y = e.take((long)N * F * 2);
@@ -554,10 +588,115 @@ struct GluBody : Body {
     const int N = e.a.n_rows;
     void* gu = e.linear(h, gate_up, N, false, false, false, nullptr);
     void* y = e.take((long)N * F * e.esize);
-    RUN(e, gibbs_glu(gu, y, e.p.dtype, N, F, act, e.a.stream));
+    if (act == ACT_CLAMPED)
+      RUN(e, gibbs_glu_clamped(gu, y, e.p.dtype, N, F, alpha, limit, e.a.stream));
+    else
+      RUN(e, gibbs_glu(gu, y, e.p.dtype, N, F, act, e.a.stream));
     e.give(gu);
     Pending delta;
     delta.data = e.linear(y, down, N, false, true, true, &delta.parts);
+    e.give(y);
+    return delta;
+  }
+};
+
+// ---- gated delta rule with short convolutions
+// One product gives [q | k | v | b | a | g] of the normed rows (segments start at multiples of 8 values); q, k, v
+// pass a short causal convolution and silu; q and k become unit vectors; the rule runs over the requests' states
+// S [heads, D, V]; each head's read-out is divided by its root mean square, multiplied by a gain and a gate, and
+// projected back.  The decay is one per head (a: heads values) or one per head and key channel (a: a low-rank
+// pair, a1 inside the product and a2 after it); the gate is silu of a full projection or sigmoid of a low-rank pair.
+struct DeltaBody : Body {
+  Matrix in, out, a2, g2;            // a2 / g2: the second matrices of the low-rank pairs (w null: none)
+  int H = 0, G = 0, D = 0, V = 0, K = 0;
+  int off_b = 0, off_a = 0, off_g = 0;   // where b, a (or a1) and g (or g1) start in a projected row
+  const float* taps = nullptr;       // [2 G D + H V, K]
+  const float* dt_bias = nullptr;
+  const float* a_log = nullptr;
+  const float* gain = nullptr;       // [V]
+  float* conv_state = nullptr;       // [slots][K - 1][2 G D + H V]
+  float* rule_state = nullptr;       // [slots][H][D][V]
+  long slot_stride = 0;
+  float eps = 0.f, unit_eps = 0.f, q_scale = 0.f;
+  Pending general(Exec& e, void* h) const override {
+    const GibbsStepArgs& a = e.a;
+    const int N = a.n_rows, C = 2 * G * D + H * V;
+    const bool channel = a2.w != nullptr;
+    char* raw = (char*)e.linear(h, in, N, false, false, false, nullptr);
+    float* qkv = (float*)e.take((long)N * C * 4);
+    RUN(e, gibbs_causal_conv_silu(raw, in.O, e.p.dtype, taps, conv_state, slot_stride, a.row_req, a.cu, a.slot, qkv, N, a.n_req, C, K, 1,
+                                  a.stream));
+    float* a_channel = channel ? (float*)e.linear(raw + (long)off_a * e.esize, a2, N, true, false, false, nullptr, in.O) : nullptr;
+    float* beta = (float*)e.take((long)N * H * 4);
+    float* decay = (float*)e.take((long)N * H * (channel ? D : 1) * 4);
+    RUN(e, gibbs_delta_prep(qkv, qkv + (long)G * D, C, raw + (long)off_b * e.esize, raw + (long)off_a * e.esize, in.O, e.p.dtype, a_channel,
+                            dt_bias, a_log, beta, decay, N, G, H, D, q_scale, unit_eps, a.stream));
+    e.give(a_channel);
+    float* o = (float*)e.take((long)N * H * V * 4);
+    RUN(e, gibbs_delta_rule(qkv, qkv + (long)G * D, C, qkv + 2L * G * D, C, beta, decay, channel, rule_state, slot_stride, a.cu, a.slot, o,
+                            a.n_req, H, G, D, V, a.stream));
+    e.give(qkv);
+    e.give(beta);
+    e.give(decay);
+    void* gate = g2.w ? e.linear(raw + (long)off_g * e.esize, g2, N, false, false, false, nullptr, in.O) : nullptr;
+    void* y = e.take((long)N * H * V * e.esize);
+    RUN(e, gibbs_head_norm_gate(o, gain, V, gate ? gate : raw + (long)off_g * e.esize, gate ? (long)H * V : in.O, y, e.p.dtype, N, H, V, eps,
+                                g2.w ? 1 : 0, a.stream));
+    e.give(gate);
+    e.give(o);
+    e.give(raw);
+    Pending delta;
+    delta.data = e.linear(y, out, N, false, true, true, &delta.parts);
+    e.give(y);
+    return delta;
+  }
+};
+
+// ---- time mixing with a decayed outer-product state
+// Each of r, k, v, g, w reads its own mix of the row and the row before it, h + (h' - h) mu_s; the decay is
+// w = exp(-exp(W2 tanh(W1 mix_w) + w0)); the rule runs over the requests' states S [heads, D, D]; each head's
+// read-out is divided by its root mean square, multiplied by a gain and silu(g), and projected back.
+struct TimeMixBody : Body {
+  Matrix wr, wk, wv, wg, w1, w2, out;
+  int H = 0, D = 0;
+  const float* mu = nullptr;         // [5, hidden]: r, k, v, g, w
+  const float* w0 = nullptr;         // [H D]
+  const float* bonus = nullptr;      // [H, D]
+  const float* gain = nullptr;       // [H D]
+  float* shift_state = nullptr;      // [slots][hidden]: the previous token's normed row
+  float* rule_state = nullptr;       // [slots][H][D][D]
+  long slot_stride = 0;
+  float eps = 0.f;
+  Pending general(Exec& e, void* h) const override {
+    const GibbsStepArgs& a = e.a;
+    const int N = a.n_rows, W = e.p.hidden, C = H * D;
+    char* mixes = (char*)e.take(5L * N * W * e.esize);
+    RUN(e, gibbs_token_shift(h, e.p.dtype, mu, 5, shift_state, slot_stride, a.row_req, a.cu, a.slot, mixes, N, a.n_req, W, 1, a.stream));
+    const long one = (long)N * W * e.esize;
+    void* r = e.linear(mixes, wr, N, false, false, false, nullptr);
+    void* k = e.linear(mixes + one, wk, N, false, false, false, nullptr);
+    void* v = e.linear(mixes + 2 * one, wv, N, false, false, false, nullptr);
+    void* g = e.linear(mixes + 3 * one, wg, N, false, false, false, nullptr);
+    float* z = (float*)e.linear(mixes + 4 * one, w1, N, true, false, false, nullptr);
+    e.give(mixes);
+    void* t = e.take((long)N * w1.O * e.esize);
+    RUN(e, gibbs_tanh_rows(z, t, e.p.dtype, (long)N * w1.O, a.stream));
+    e.give(z);
+    float* w = (float*)e.linear(t, w2, N, true, false, false, nullptr);
+    e.give(t);
+    RUN(e, gibbs_double_exp_decay(w, w0, (long)N * C, C, a.stream));
+    float* o = (float*)e.take((long)N * C * 4);
+    RUN(e, gibbs_decayed_outer_rule(r, k, v, e.p.dtype, w, bonus, rule_state, slot_stride, a.cu, a.slot, o, a.n_req, H, D, a.stream));
+    e.give(r);
+    e.give(k);
+    e.give(v);
+    e.give(w);
+    void* y = e.take((long)N * C * e.esize);
+    RUN(e, gibbs_head_norm_gate(o, gain, C, g, C, y, e.p.dtype, N, H, D, eps, 0, a.stream));
+    e.give(o);
+    e.give(g);
+    Pending delta;
+    delta.data = e.linear(y, out, N, false, true, true, &delta.parts);
     e.give(y);
     return delta;
   }
@@ -583,10 +722,13 @@ void Exec::run() {
   const int N = a.n_rows, H = p.hidden;
   float* x = a.x_in;
   void* mirror = few_rows ? a.mirror_in : nullptr;
+  float* embedded = nullptr;     // the embedding's output, for a program that adds it again
   if (!x) {
     x = (float*)take((long)N * H * 4);
     mirror = few_rows ? take((long)N * H * 2) : nullptr;
-    RUN(*this, gibbs_embed(p.table, p.table_dtype, a.ids, x, mirror, N, H, p.vocab, a.stream));
+    if (p.reinjects) embedded = (float*)take((long)N * H * 4);
+    RUN(*this, gibbs_embed_general(p.table, p.table_dtype, a.ids, x, mirror, N, H, p.vocab, p.embed_scale, a.pos, p.embed_inv_freq,
+                                   embedded, a.stream));
   }
   Pending pending;
   std::vector<void*> rows(p.n_values, nullptr);       // normed rows by value
@@ -626,6 +768,17 @@ void Exec::run() {
         pending = deltas[op.value];
         deltas[op.value] = Pending{};
         break;
+      case Plan::OP_NORM_DELTA:
+        deltas[op.result] = p.norms[op.norm]->run_on(*this, deltas[op.value]);
+        deltas[op.value] = Pending{};
+        break;
+      case Plan::OP_REINJECT:
+        settle(x, pending);
+        if (!embedded) { if (!status) status = gibbs_fail("step: the embedding's output is added again, but the caller brought the rows"); break; }
+        RUN(*this, gibbs_residual_add(x, embedded, GIBBS_F32, 1, (long)N * H, nullptr, (long)N * H, a.stream));
+        give(mirror);
+        mirror = nullptr;
+        break;
       case Plan::OP_DROP:
         give(rows[op.value]);
         give(deltas[op.value].data);
@@ -644,6 +797,7 @@ void Exec::run() {
   for (void* r : rows) give(r);
   for (Pending& d : deltas) give(d.data);
   give(mirror);      // (buffers of the caller's are not the arena's: giving them back does nothing)
+  give(embedded);
   give(x);
 }
 
@@ -656,6 +810,7 @@ int check_args(const Plan* p, const GibbsStepArgs* a, bool whole_step) {
   GIBBS_REQUIRE(a->lead_single >= 0 && a->lead_single <= a->n_req, "step: %d leading decoded tokens among %d requests", a->lead_single, a->n_req);
   GIBBS_REQUIRE(a->first_op >= 0 && a->n_ops >= 0 && a->first_op + a->n_ops <= (int)p->ops.size(), "step: operations %d .. %d of %d", a->first_op, a->first_op + a->n_ops, (int)p->ops.size());
   GIBBS_REQUIRE(a->x_in || p->table, "step: the plan has no token table and the caller brought no rows");
+  GIBBS_REQUIRE(!a->x_in || !p->reinjects || a->n_ops, "step: this model adds its embedding's output again: the step embeds its rows itself");
   if (a->n_ops == 0 && a->n_logits > 0) {
     GIBBS_REQUIRE(p->has_norm(p->tail) && p->head.w, "step: logits are wanted and the plan has no final norm or no head");
     GIBBS_REQUIRE(a->workspace == nullptr || a->logits, "step: logits are wanted and there is no buffer for them");
@@ -744,7 +899,7 @@ GIBBS_EXPORT int gibbs_plan_body_attention(void* plan, const void* w_qkv, const 
   t->nh = nh; t->nkv = nkv; t->hd = hd; t->scale = scale; t->window = window; t->q_gain = q_gain; t->k_gain = k_gain; t->qk_eps = qk_eps;
   t->inv_freq = inv_freq; t->rot = inv_freq ? rot : 0; t->variant = variant; t->cos_sin = cos_sin; t->table_len = table_len;
   t->kpages = kpages; t->vpages = vpages; t->num_pages = num_pages; t->page_size = page_size; t->group = group; t->owns = owns;
-  t->slopes = slopes; t->hook = hook; t->hook_user = hook_user;
+  t->slopes = slopes; t->hook = hook; t->hook_user = hook_user; t->vd = hd;
   p->bodies.push_back(std::move(t));
   return (int)p->bodies.size() - 1;
 }
@@ -771,6 +926,90 @@ GIBBS_EXPORT int gibbs_plan_body_host(void* plan, GibbsHostBody fn, void* user, 
   if (!fn) { gibbs_fail("plan: a body from elsewhere needs its function"); return -1; }
   auto b = std::make_unique<HostBody>();
   b->fn = fn; b->user = user; b->group = group;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+// ---- more about parts that are there already
+GIBBS_EXPORT int gibbs_plan_embedding(void* plan, float scale, const float* inv_freq) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  p->embed_scale = scale; p->embed_inv_freq = inv_freq;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, float temp_coef, int temp_every,
+                                             const float* bias, int bias_len) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  AttnBody* t = p->has_body(body) ? dynamic_cast<AttnBody*>(p->bodies[body].get()) : nullptr;
+  if (!t || vd <= 0 || temp_every < 0 || (bias && bias_len <= 0)) { gibbs_fail("plan: body %d is no attention, or bad extras", body); return -1; }
+  if (t->inv_freq || t->q_gain || t->k_gain || t->hook || t->slopes || !t->owns) {
+    gibbs_fail("plan: an attention with these extras has no rotation, no q/k gains, no hook and no slopes, and owns its pages");
+    return -1;
+  }
+  t->vd = vd; t->unit_qk = unit_qk; t->temp_coef = temp_coef; t->temp_every = temp_every; t->bias = bias; t->bias_len = bias ? bias_len : 0;
+  t->qkv.O = (t->nh + t->nkv) * t->hd + t->nkv * vd;
+  t->out.I = t->nh * vd;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_glu_clamped(void* plan, int body, float alpha, float limit) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  GluBody* g = p->has_body(body) ? dynamic_cast<GluBody*>(p->bodies[body].get()) : nullptr;
+  if (!g || !(limit > 0.f)) { gibbs_fail("plan: body %d is no gated feed-forward, or its limit is not positive", body); return -1; }
+  g->act = ACT_CLAMPED; g->alpha = alpha; g->limit = limit;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_delta(void* plan, const GibbsDeltaSpec* d) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!d || !(d->w_in && d->w_out && d->taps && d->dt_bias && d->a_log && d->gain && d->conv_state && d->rule_state && d->heads > 0 &&
+              d->kv_heads > 0 && d->heads % d->kv_heads == 0 && d->dim > 0 && d->dim <= 256 && d->vdim > 0 && d->taps_per_channel >= 1 &&
+              d->in_rows > 0 && d->off_b >= 0 && d->off_a >= 0 && d->off_g >= 0 && (!d->w_a2 || d->a_rank > 0) && (!d->w_g2 || d->g_rank > 0))) {
+    gibbs_fail("plan: bad delta-rule mixer");
+    return -1;
+  }
+  const int C = 2 * d->kv_heads * d->dim + d->heads * d->vdim;
+  if (d->slot_stride < (long)d->heads * d->dim * d->vdim || d->slot_stride < (long)(d->taps_per_channel - 1) * C) {
+    gibbs_fail("plan: a state slot of %ld floats is too small for the delta-rule mixer", d->slot_stride);
+    return -1;
+  }
+  auto b = std::make_unique<DeltaBody>();
+  b->in = Matrix{d->w_in, nullptr, d->in_rows, p->hidden};
+  b->out = Matrix{d->w_out, nullptr, p->hidden, d->heads * d->vdim};
+  if (d->w_a2) b->a2 = Matrix{d->w_a2, nullptr, d->heads * d->dim, d->a_rank};
+  if (d->w_g2) b->g2 = Matrix{d->w_g2, nullptr, d->heads * d->vdim, d->g_rank};
+  b->H = d->heads; b->G = d->kv_heads; b->D = d->dim; b->V = d->vdim; b->K = d->taps_per_channel;
+  b->off_b = d->off_b; b->off_a = d->off_a; b->off_g = d->off_g;
+  b->taps = d->taps; b->dt_bias = d->dt_bias; b->a_log = d->a_log; b->gain = d->gain;
+  b->conv_state = d->conv_state; b->rule_state = d->rule_state; b->slot_stride = d->slot_stride;
+  b->eps = d->eps; b->unit_eps = d->unit_eps; b->q_scale = d->q_scale;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_time_mix(void* plan, const GibbsTimeMixSpec* d) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!d || !(d->w_r && d->w_k && d->w_v && d->w_g && d->w_1 && d->w_2 && d->w_out && d->mu && d->w0 && d->bonus && d->gain &&
+              d->shift_state && d->rule_state && d->heads > 0 && d->dim > 0 && d->dim <= 256 && d->rank > 0)) {
+    gibbs_fail("plan: bad time-mixing mixer");
+    return -1;
+  }
+  if (d->slot_stride < (long)d->heads * d->dim * d->dim || d->slot_stride < p->hidden) {
+    gibbs_fail("plan: a state slot of %ld floats is too small for the time-mixing mixer", d->slot_stride);
+    return -1;
+  }
+  const int C = d->heads * d->dim, W = p->hidden;
+  auto b = std::make_unique<TimeMixBody>();
+  b->wr = Matrix{d->w_r, nullptr, C, W}; b->wk = Matrix{d->w_k, nullptr, C, W}; b->wv = Matrix{d->w_v, nullptr, C, W};
+  b->wg = Matrix{d->w_g, nullptr, C, W}; b->w1 = Matrix{d->w_1, nullptr, d->rank, W}; b->w2 = Matrix{d->w_2, nullptr, C, d->rank};
+  b->out = Matrix{d->w_out, nullptr, W, C};
+  b->H = d->heads; b->D = d->dim; b->mu = d->mu; b->w0 = d->w0; b->bonus = d->bonus; b->gain = d->gain;
+  b->shift_state = d->shift_state; b->rule_state = d->rule_state; b->slot_stride = d->slot_stride; b->eps = d->eps;
   p->bodies.push_back(std::move(b));
   return (int)p->bodies.size() - 1;
 }
@@ -814,6 +1053,18 @@ GIBBS_EXPORT int gibbs_plan_op_drop(void* plan, int value) {
   if (!p) return -1;
   if (!known_value(p, value)) { gibbs_fail("plan: no value %d to drop", value); return -1; }
   return append(p, Plan::OP_DROP, -1, -1, value, false);
+}
+GIBBS_EXPORT int gibbs_plan_op_norm_delta(void* plan, int norm, int value) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!p->has_norm(norm) || !known_value(p, value)) { gibbs_fail("plan: norm %d of value %d: no such part or value", norm, value); return -1; }
+  return append(p, Plan::OP_NORM_DELTA, norm, -1, value, true);
+}
+GIBBS_EXPORT int gibbs_plan_op_reinject(void* plan) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  p->reinjects = true;
+  return append(p, Plan::OP_REINJECT, -1, -1, -1, false);
 }
 GIBBS_EXPORT int gibbs_plan_tail(void* plan, int norm) {
   Plan* p = open_plan(plan);

@@ -71,12 +71,51 @@ int gibbs_plan_body_glu(void* plan, const void* w_gate_up, const void* p_gate_up
                         int F, int act);
 int gibbs_plan_body_host(void* plan, GibbsHostBody fn, void* user, int group);   // group: the cache group it reads, or -1
 
+// The embedding: rows of the table times `scale`, plus (inv_freq [hidden / 2] not null) a sinusoidal position vector,
+// entry 2i = sin(pos * inv_freq[i]), entry 2i + 1 = cos of the same.
+int gibbs_plan_embedding(void* plan, float scale, const float* inv_freq);
+// An attention body without rotation and q/k gains may have: values of head size vd; q and k divided by their root
+// mean square per head (unit_qk, with the body's qk_eps); q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)
+// (temp_every 0: none); bias [bias_len, heads] added to the scores by distance (the last row for all longer ones).
+// Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd].
+int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, float temp_coef, int temp_every, const float* bias,
+                                int bias_len);
+// A gated feed-forward body computes min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1) instead.
+int gibbs_plan_glu_clamped(void* plan, int body, float alpha, float limit);
+
+// Gated delta rule with short convolutions.  w_in [in_rows, hidden]: the rows of q (kv_heads*dim), k (the same), v
+// (heads*vdim), then at off_b the heads rows of beta's projection, at off_a the decay's (heads rows, or a_rank rows of
+// the first matrix of a low-rank pair whose second is w_a2 [heads*dim, a_rank]: one decay per key channel), at off_g the
+// gate's (heads*vdim rows and silu, or g_rank rows and w_g2 [heads*vdim, g_rank] and sigmoid).  taps [2 kv_heads dim +
+// heads vdim, taps_per_channel], the last one the current token's.
+struct GibbsDeltaSpec {
+  const void* w_in; const void* w_out; const void* w_a2; const void* w_g2;
+  const float* taps; const float* dt_bias; const float* a_log; const float* gain;
+  float* conv_state; float* rule_state; long slot_stride;
+  int in_rows, heads, kv_heads, dim, vdim, taps_per_channel, off_b, off_a, off_g, a_rank, g_rank;
+  float eps, unit_eps, q_scale;
+};
+int gibbs_plan_body_delta(void* plan, const struct GibbsDeltaSpec* spec);
+
+// Time mixing with a decayed outer-product state.  w_r, w_k, w_v, w_g [heads*dim, hidden], w_1 [rank, hidden], w_2
+// [heads*dim, rank], w_out [hidden, heads*dim]; mu [5, hidden] (r, k, v, g, w); w0, gain [heads*dim]; bonus [heads, dim].
+struct GibbsTimeMixSpec {
+  const void* w_r; const void* w_k; const void* w_v; const void* w_g; const void* w_1; const void* w_2; const void* w_out;
+  const float* mu; const float* w0; const float* bonus; const float* gain;
+  float* shift_state; float* rule_state; long slot_stride;
+  int heads, dim, rank;
+  float eps;
+};
+int gibbs_plan_body_time_mix(void* plan, const struct GibbsTimeMixSpec* spec);
+
 // ---- the program (values are normed rows or deltas, named by the index their operation returns)
 int gibbs_plan_op_half(void* plan, int norm, int body);       // x += body(norm(x)), in fused kernels where it can
 int gibbs_plan_op_norm(void* plan, int norm);                 // -> value: norm(x + what is pending)
 int gibbs_plan_op_body(void* plan, int body, int value);      // -> value: body(normed rows)
 int gibbs_plan_op_add(void* plan, int value);                 // x += delta (lazily: it stays pending for the next norm)
 int gibbs_plan_op_drop(void* plan, int value);                // the value is not read again
+int gibbs_plan_op_norm_delta(void* plan, int norm, int value);   // -> value: norm(a body's delta), the stream untouched
+int gibbs_plan_op_reinject(void* plan);                       // x += the embedding's output (what the step's first operation saw)
 int gibbs_plan_tail(void* plan, int norm);                    // the norm in front of the head
 int gibbs_plan_op_count(const void* plan);
 

@@ -99,9 +99,13 @@ class DecodeLoop:
         self.live_mask = torch.zeros(b, dtype=torch.int32, device=dev) if self.padded else None   # 0: a row of padding
         # native step: the rows of the residual stream (and their bfloat16 mirror) live here from one step to
         # the next; the end of a step writes the next tokens' embeddings into them
+        # (a model whose embedding is more than the table's rows, a scale, a position vector, rows that come back
+        # later in the step, embeds the ids itself at the start of every step: the end of a step then only
+        # leaves the sampled ids and the advanced positions)
         hidden = engine.spec.hidden
-        self.x = torch.zeros((b, hidden), dtype=torch.float32, device=dev)
-        self.mirror = torch.zeros((b, hidden), dtype=torch.bfloat16, device=dev) if engine.dtype == torch.bfloat16 else None
+        self.x = torch.zeros((b, hidden), dtype=torch.float32, device=dev) if engine.plan.plain_embedding else None
+        self.mirror = (torch.zeros((b, hidden), dtype=torch.bfloat16, device=dev)
+                       if engine.dtype == torch.bfloat16 and self.x is not None else None)
         if not self.greedy:
             self.temperature = torch.zeros(b, dtype=torch.float32, device=dev)
             self.top_p = torch.zeros(b, dtype=torch.float32, device=dev)
@@ -166,7 +170,8 @@ class DecodeLoop:
     def _embed(self) -> None:
         """The embeddings of the tokens in `ids` into the loop's residual rows (the first step after binding;
         every later step finds what the end of the step before it wrote)."""
-        ops.embed(self.engine.model.table, self.batch.ids, self.n, out=self.x, mirror=self.mirror)
+        if self.x is not None:
+            ops.embed(self.engine.model.table, self.batch.ids, self.n, out=self.x, mirror=self.mirror)
 
     # ------------------------------------------------------------------ host side
     def _fill_tables(self) -> None:

@@ -37,34 +37,41 @@ class AttentionMixer(Mixer):
         self.qk_norm = p.get("qk_norm")
         self.qk_norm_eps = float(p.get("qk_norm_eps", 0.0))
         self.source = p.get("kv_source")
+        # values of a head size of their own; q and k divided by their root mean square without a gain
+        # (`qk_norm: "unit"`); q times 1 + coef * ln(floor((position + 1) / every) + 1) (`q_temperature`)
+        self.v_head_dim = int(p.get("v_head_dim") or self.head_dim)
+        self.q_temperature = p.get("q_temperature")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads are not a multiple of {self.kv_heads} kv heads")
-        if self.qk_norm not in (None, "before"):
-            raise ValueError(f"qk_norm {self.qk_norm!r} is not implemented (None or 'before')")
+        if self.qk_norm not in (None, "before", "unit"):
+            raise ValueError(f"qk_norm {self.qk_norm!r} is not implemented (None, 'before' or 'unit')")
         if self.window is not None and int(self.window) <= 0:
             raise ValueError(f"attention window {self.window} must be positive")
         self.position = build_position(spec.position, self.head_dim)
+        if hasattr(self.position, "for_heads"):          # (an encoding with a column per head)
+            self.position.for_heads(self.heads)
 
     # ------------------------------------------------------------------ what it asks for
     def cache_need(self) -> Optional[CacheNeed]:
         if self.source is not None:
             return None
-        return CacheNeed(self.kv_heads, self.head_dim, None if self.window is None else int(self.window))
+        return CacheNeed(self.kv_heads, self.head_dim, None if self.window is None else int(self.window),
+                         None if self.v_head_dim == self.head_dim else self.v_head_dim)
 
     def attention_flops(self, keys: float) -> float:
         """Multiply-adds x 2 of scores and weighted values when the step's rows see `keys` keys in all."""
-        return 2.0 * 2.0 * keys * self.heads * self.head_dim
+        return 2.0 * keys * self.heads * (self.head_dim + self.v_head_dim)
 
     def kv_source(self) -> Optional[int]:
         return self.source
 
     def tensor_decls(self) -> List[TensorDecl]:
-        t, H, hd = self.spec.tensors, self.hidden, self.head_dim
+        t, H, hd, vd = self.spec.tensors, self.hidden, self.head_dim, self.v_head_dim
         decls = [TensorDecl(t["q_proj"], (self.heads * hd, H))]
         if self.source is None:
-            decls += [TensorDecl(t["k_proj"], (self.kv_heads * hd, H)), TensorDecl(t["v_proj"], (self.kv_heads * hd, H))]
-        decls.append(TensorDecl(t["out_proj"], (H, self.heads * hd)))
-        if self.qk_norm:
+            decls += [TensorDecl(t["k_proj"], (self.kv_heads * hd, H)), TensorDecl(t["v_proj"], (self.kv_heads * vd, H))]
+        decls.append(TensorDecl(t["out_proj"], (H, self.heads * vd)))
+        if self.qk_norm == "before":
             decls.append(TensorDecl(t["q_norm"], (hd,), FLOAT32, init="gain"))
             if self.source is None:
                 decls.append(TensorDecl(t["k_norm"], (hd,), FLOAT32, init="gain"))
@@ -82,13 +89,14 @@ class AttentionMixer(Mixer):
             self.w_qkv = weights[t["q_proj"]]
         self.w_out = weights[t["out_proj"]]
         self.p_qkv = self.p_out = None
-        self.q_gain = weights[t["q_norm"]] if self.qk_norm else None
-        self.k_gain = weights[t["k_norm"]] if self.qk_norm and self.source is None else None
-        self.rot, self.slopes, self.pos_hook = None, None, False
+        self.q_gain = weights[t["q_norm"]] if self.qk_norm == "before" else None
+        self.k_gain = weights[t["k_norm"]] if self.qk_norm == "before" and self.source is None else None
+        self.rot, self.slopes, self.pos_hook, self.score_bias = None, None, False, None
         if self.position is not None:
             self.position.bind(weights, rt)
             self.rot = self.position.rotation()
             self.slopes = self.position.score_slopes(self.heads)
+            self.score_bias = self.position.score_table(self.heads)
             self.pos_hook = self.rot is None and self.position.transforms_rows()
         if self.slopes is not None and (self.slopes.dtype != torch.float32 or tuple(self.slopes.shape) != (self.heads,)):
             raise ValueError(f"score slopes must be float32 [{self.heads}]")
@@ -97,11 +105,11 @@ class AttentionMixer(Mixer):
         return [self.w_qkv, self.w_out]
 
     def product_shapes(self):
-        kv = 2 * self.kv_heads if self.source is None else 0
-        return [((self.heads + kv) * self.head_dim, self.hidden), (self.hidden, self.heads * self.head_dim)]
+        kv = self.kv_heads * (self.head_dim + self.v_head_dim) if self.source is None else 0
+        return [(self.heads * self.head_dim + kv, self.hidden), (self.hidden, self.heads * self.v_head_dim)]
 
     def small_tensors(self):
-        own = [t for t in (self.q_gain, self.k_gain, self.slopes) if t is not None]
+        own = [t for t in (self.q_gain, self.k_gain, self.slopes) if t is not None]   # (a score table is the position's)
         return own + ([] if self.position is None else list(self.position.small_tensors()))
 
     def fold_input_gain(self, gain: torch.Tensor) -> None:
@@ -112,10 +120,23 @@ class AttentionMixer(Mixer):
         self.p_qkv = ops.PackedWeight(self.w_qkv)
         self.p_out = ops.PackedWeight(self.w_out)
 
+    def extras(self) -> bool:
+        """Options that the plain kernels take and the matrix-core kernels do not."""
+        return (self.v_head_dim != self.head_dim or self.qk_norm == "unit" or self.q_temperature is not None
+                or self.score_bias is not None)
+
     def emit(self, plan, cache) -> int:
-        if cache.kpages is None or cache.kpages.shape != cache.vpages.shape:
-            raise ValueError("the attention mixer's kernels want keys and values of one head size")
+        if cache.kpages is None or cache.vpages.shape[-1] != self.v_head_dim or cache.kpages.shape[-1] != self.head_dim:
+            raise ValueError("the attention mixer's pages do not have its head sizes")
         hook = self.position.apply if self.pos_hook else None
+        body = self._emit_body(plan, cache, hook)
+        if self.extras():
+            temp = self.q_temperature or {"coef": 0.0, "every": 0}
+            plan.attention_extras(body, v_head_dim=self.v_head_dim, unit_qk=self.qk_norm == "unit", temp_coef=float(temp["coef"]),
+                                  temp_every=int(temp["every"]), bias=self.score_bias)
+        return body
+
+    def _emit_body(self, plan, cache, hook) -> int:
         return plan.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
                               kv_heads=self.kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
                               q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,

@@ -124,7 +124,8 @@ class PositionEncoding(Part):
       apply(q, k, batch)  anything else done to q and k in place before k is cached (the mixer then
                         takes its general path: norm, this hook, cache write, attention);
       score_slopes(heads)  float32 [heads]: slope[h] * (key position - query position) is added to the
-                        scores (a linear bias over the distance; the plain attention kernel takes it).
+                        scores (a linear bias over the distance; the plain attention kernel takes it);
+      score_table(heads)  float32 [distances, heads]: any bias over the distance, as a table.
 
     An encoding that answers none of them leaves q, k and the scores alone."""
 
@@ -140,6 +141,11 @@ class PositionEncoding(Part):
         holds every row's position."""
 
     def score_slopes(self, heads: int) -> Optional[torch.Tensor]:
+        return None
+
+    def score_table(self, heads: int) -> Optional[torch.Tensor]:
+        """float32 [distances, heads]: row n is added to the scores of keys n positions back, the last row to
+        those of all keys farther back (any bias over the distance; the plain attention kernel takes it)."""
         return None
 
     def transforms_rows(self) -> bool:

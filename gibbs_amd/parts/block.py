@@ -47,3 +47,47 @@ class PreNormBlock(Block):
     def emit(self, plan, caches) -> None:
         plan.half(self.mixer_norm.emit(plan), self.mixer.emit(plan, caches["mixer"]))
         plan.half(self.ffn_norm.emit(plan), self.ffn.emit(plan))
+
+
+@register_arrangement("parallel_norms")
+class ParallelNormsBlock(Block):
+    """Mixer and feed-forward side by side, each on a norm of its own of the same stream:
+
+        x = x + mixer(norm1(x)) + ffn(norm2(x))
+
+    Roles: `norm1`, then either `mixer`, or a pair of mixers `left` and `right` that read the same normed rows,
+    each result normed over the width by `left_out` / `right_out` and the two averaged; `norm2` and `ffn` may
+    be missing (a layer without a feed-forward).  The average's half is multiplied into the two out-norms'
+    gains when the weights are bound (exact: a power of two).  No gain is folded into matrices and no half of
+    this block takes the fused decode kernels: the step runs norm, body and add operations."""
+
+    def __init__(self, spec, hidden, layer_index):
+        super().__init__(spec, hidden, layer_index)
+        self.pair = "left" in self.named
+        want = ["norm1"] + (["left", "right", "left_out", "right_out"] if self.pair else ["mixer"])
+        want += ["norm2"] if "ffn" in self.named else []
+        missing = [r for r in want if r not in self.named]
+        if missing:
+            raise ValueError(f"layer {spec.name!r} lacks the parts {missing}")
+
+    def bind(self, weights, rt: Runtime) -> None:
+        super().bind(weights, rt)
+        if self.pair:
+            for norm in (self.left_out, self.right_out):
+                norm.gain = norm.gain * 0.5
+
+    def emit(self, plan, caches) -> None:
+        h = plan.normed(self.norm1.emit(plan))
+        if self.pair:
+            left = plan.apply(self.left.emit(plan, caches["left"]), h)
+            right = plan.apply(self.right.emit(plan, caches["right"]), h)
+            deltas = [plan.normed_delta(self.left_out.emit(plan), left), plan.normed_delta(self.right_out.emit(plan), right)]
+        else:
+            deltas = [plan.apply(self.mixer.emit(plan, caches["mixer"]), h)]
+        plan.drop(h)
+        if "ffn" in self.named:
+            h2 = plan.normed(self.norm2.emit(plan))
+            deltas.append(plan.apply(self.ffn.emit(plan), h2))
+            plan.drop(h2)
+        for d in deltas:
+            plan.add(d)

@@ -1,6 +1,9 @@
 """Dense gated feed-forward: down(act(gate(h)) * up(h)), `activation` one of `ops.ACTIVATIONS`; with "silu" this is
 SwiGLU (arch/lib/transformer.json5:117-130, src/graph/cpu.rs:378-390).
-Gate and up are one product against [W_gate; W_up]."""
+Gate and up are one product against [W_gate; W_up].
+
+`activation: "clamped_swish"` (with `limit` and `alpha`) is the clamped variant: g = min(gate, limit), u =
+clamp(up, -limit, limit), down(g * sigmoid(alpha * g) * (u + 1))."""
 from __future__ import annotations
 
 from typing import List
@@ -18,7 +21,12 @@ class GluFeedForward(FeedForward):
         super().__init__(spec, hidden)
         self.inter = int(spec.params["inter"])
         self.activation = spec.params.get("activation", "silu")
-        if self.activation not in ops.ACTIVATIONS:
+        self.clamped = self.activation == "clamped_swish"
+        if self.clamped:
+            self.limit, self.alpha = float(spec.params["limit"]), float(spec.params.get("alpha", 1.702))
+            if not self.limit > 0:
+                raise ValueError(f"the clamped feed-forward's limit {self.limit} must be positive")
+        elif self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"feed-forward activation {self.activation!r} is not implemented")
 
     def tensor_decls(self) -> List[TensorDecl]:
@@ -48,5 +56,8 @@ class GluFeedForward(FeedForward):
         self.p_down = ops.PackedWeight(self.w_down)
 
     def emit(self, plan) -> int:
-        return plan.glu(w_gate_up=self.w_gate_up, p_gate_up=self.p_gate_up, w_down=self.w_down, p_down=self.p_down,
-                        inter=self.inter, activation=ops.ACTIVATIONS[self.activation])
+        body = plan.glu(w_gate_up=self.w_gate_up, p_gate_up=self.p_gate_up, w_down=self.w_down, p_down=self.p_down,
+                        inter=self.inter, activation=0 if self.clamped else ops.ACTIVATIONS[self.activation])
+        if self.clamped:
+            plan.glu_clamped(body, alpha=self.alpha, limit=self.limit)
+        return body

@@ -24,6 +24,8 @@ class DecoderModel(Part):
         self.spec = spec
         self.blocks: List[Block] = [build_block(ls, spec.hidden, i) for i, ls in enumerate(spec.layers)]
         self.final_norm = build_norm(spec.final_norm, spec.hidden)
+        if any(not 0 < r < len(spec.order) for r in spec.reinject_before):
+            raise ValueError(f"the embedding's output is added again before runs {list(spec.reinject_before)}; the order has {len(spec.order)}")
         for i in spec.order:
             if not 0 <= i < len(self.blocks):
                 raise ValueError(f"layer order names layer {i}; the model has {len(self.blocks)}")
@@ -88,6 +90,15 @@ class DecoderModel(Part):
         self.table = weights[self.spec.embedding]
         self.head = weights[self.spec.head] if self.spec.head is not None else self.table
         self.head_packed = ops.PackedWeight(self.head) if rt.act_dtype == torch.bfloat16 else None
+        self.embedding_inv_freq = None
+        pos = self.spec.embedding_position
+        if pos is not None and pos.kind != "none":
+            if pos.kind != "sinusoidal":
+                raise ValueError(f"position vector of kind {pos.kind!r} on the embedding is not implemented ('sinusoidal')")
+            # entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i) with f_i = base^(-2i / width), rounded to float32 once
+            width = self.spec.hidden
+            i = torch.arange(width // 2, dtype=torch.float64)
+            self.embedding_inv_freq = (float(pos.params.get("base", 10000.0)) ** (-2.0 * i / width)).to(torch.float32).to(rt.device)
         self.final_norm.bind(weights, rt)
         for b in self.blocks:
             b.bind(weights, rt)

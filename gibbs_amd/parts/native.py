@@ -34,6 +34,24 @@ class StepArgs(ctypes.Structure):
                 ("first_op", c_int), ("n_ops", c_int), ("settle", c_int)]
 
 
+class DeltaSpec(ctypes.Structure):
+    """GibbsDeltaSpec of csrc/step_plan_api.h."""
+    _fields_ = [("w_in", c_void_p), ("w_out", c_void_p), ("w_a2", c_void_p), ("w_g2", c_void_p),
+                ("taps", c_void_p), ("dt_bias", c_void_p), ("a_log", c_void_p), ("gain", c_void_p),
+                ("conv_state", c_void_p), ("rule_state", c_void_p), ("slot_stride", c_long),
+                ("in_rows", c_int), ("heads", c_int), ("kv_heads", c_int), ("dim", c_int), ("vdim", c_int),
+                ("taps_per_channel", c_int), ("off_b", c_int), ("off_a", c_int), ("off_g", c_int), ("a_rank", c_int),
+                ("g_rank", c_int), ("eps", ctypes.c_float), ("unit_eps", ctypes.c_float), ("q_scale", ctypes.c_float)]
+
+
+class TimeMixSpec(ctypes.Structure):
+    """GibbsTimeMixSpec of csrc/step_plan_api.h."""
+    _fields_ = [("w_r", c_void_p), ("w_k", c_void_p), ("w_v", c_void_p), ("w_g", c_void_p), ("w_1", c_void_p), ("w_2", c_void_p),
+                ("w_out", c_void_p), ("mu", c_void_p), ("w0", c_void_p), ("bonus", c_void_p), ("gain", c_void_p),
+                ("shift_state", c_void_p), ("rule_state", c_void_p), ("slot_stride", c_long),
+                ("heads", c_int), ("dim", c_int), ("rank", c_int), ("eps", ctypes.c_float)]
+
+
 HOST_BODY = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p)
 HOST_NORM = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p)
 HOST_ROWS = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_long)
@@ -56,6 +74,13 @@ def declare(lib) -> None:
         "gibbs_plan_body_attention": ([P, P, P, P, P, I, I, I, F, I, P, P, F, P, I, I, P, I, P, P, I, I, I, I, P, HOST_ROWS, P], I),
         "gibbs_plan_body_glu": ([P, P, P, P, P, I, I], I),
         "gibbs_plan_body_host": ([P, HOST_BODY, P, I], I),
+        "gibbs_plan_embedding": ([P, F, P], I),
+        "gibbs_plan_attention_extras": ([P, I, I, I, F, I, P, I], I),
+        "gibbs_plan_glu_clamped": ([P, I, F, F], I),
+        "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
+        "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
+        "gibbs_plan_op_norm_delta": ([P, I, I], I),
+        "gibbs_plan_op_reinject": ([P], I),
         "gibbs_plan_op_half": ([P, I, I], I),
         "gibbs_plan_op_norm": ([P, I], I),
         "gibbs_plan_op_body": ([P, I, I], I),
@@ -105,6 +130,8 @@ class NativePlan:
         self._workspace: Optional[torch.Tensor] = None
         self._x_in: Optional[torch.Tensor] = None
         self._error: Optional[BaseException] = None
+        # the rows of a step are the table's rows and nothing else (a caller may then bring them itself, `x_in`)
+        self.plain_embedding = True
 
     def __del__(self):
         if getattr(self, "handle", None):
@@ -169,7 +196,7 @@ class NativePlan:
             inv_freq, cos_sin, rot = rotation.inv_freq, rotation.cos_sin, int(rotation.rotary_dim)
             variant = ROPE_VARIANTS[rotation.variant]
             table_len = 0 if cos_sin is None else int(cos_sin.shape[0])
-        assert kpages.is_contiguous() and vpages.is_contiguous() and kpages.shape == vpages.shape
+        assert kpages.is_contiguous() and vpages.is_contiguous() and kpages.shape[:-1] == vpages.shape[:-1]
         ptrs = self._held(w_qkv, p_qkv, w_out, p_out)
         gains = self._held(q_gain, k_gain)
         tables = self._held(inv_freq, cos_sin)
@@ -200,6 +227,47 @@ class NativePlan:
     def glu(self, *, w_gate_up, p_gate_up, w_down, p_down, inter: int, activation: int) -> int:
         ptrs = self._held(w_gate_up, p_gate_up, w_down, p_down)
         return self._made(L.library().gibbs_plan_body_glu(self.handle, *ptrs, int(inter), int(activation)))
+
+    def attention_extras(self, body: int, *, v_head_dim: int, unit_qk: bool, temp_coef: float, temp_every: int, bias) -> None:
+        """Options of an attention body without rotation: values of a head size of their own, q and k divided by
+        their root mean square, a temperature on q, a table [distances, heads] of score biases."""
+        (b,) = self._held(bias)
+        self._made(L.library().gibbs_plan_attention_extras(self.handle, int(body), int(v_head_dim), int(unit_qk), float(temp_coef),
+                                                           int(temp_every), b, 0 if bias is None else int(bias.shape[0])))
+
+    def glu_clamped(self, body: int, *, alpha: float, limit: float) -> None:
+        self._made(L.library().gibbs_plan_glu_clamped(self.handle, int(body), float(alpha), float(limit)))
+
+    def embedding(self, scale: float, inv_freq: Optional[torch.Tensor]) -> None:
+        """The table's rows times `scale`, plus the sinusoidal position vector of `inv_freq` (float32 [hidden / 2])."""
+        (f,) = self._held(inv_freq)
+        self._made(L.library().gibbs_plan_embedding(self.handle, float(scale), f))
+        self.plain_embedding = self.plain_embedding and scale == 1.0 and inv_freq is None
+
+    def gated_delta(self, m, *, conv_state: torch.Tensor, rule_state: torch.Tensor) -> int:
+        """The delta-rule mixer `m` (parts/delta.py) over its states [slots, ...] in the arena."""
+        assert rule_state.dtype == torch.float32 and conv_state.dtype == torch.float32 and rule_state.stride(0) == conv_state.stride(0)
+        d = DeltaSpec()
+        d.w_in, d.w_out, d.w_a2, d.w_g2 = self._held(m.w_in, m.w_out, m.w_a2, m.w_g2)
+        d.taps, d.dt_bias, d.a_log, d.gain = self._held(m.conv_taps, m.dt_bias, m.a_log, m.gain)
+        d.conv_state, d.rule_state, d.slot_stride = conv_state.data_ptr(), rule_state.data_ptr(), int(rule_state.stride(0))
+        self.keep += [conv_state, rule_state]
+        d.in_rows, d.heads, d.kv_heads, d.dim, d.vdim = m.w_in.shape[0], m.heads, m.kv_heads, m.dim, m.vdim
+        d.taps_per_channel, d.off_b, d.off_a, d.off_g = m.taps, m.off_b, m.off_a, m.off_g
+        d.a_rank, d.g_rank = m.decay_rank, m.gate_rank
+        d.eps, d.unit_eps, d.q_scale = m.norm_eps, m.unit_eps, m.q_scale
+        return self._made(L.library().gibbs_plan_body_delta(self.handle, ctypes.byref(d)))
+
+    def time_mix(self, m, *, shift_state: torch.Tensor, rule_state: torch.Tensor) -> int:
+        """The time-mixing mixer `m` (parts/timemix.py) over its states [slots, ...] in the arena."""
+        assert rule_state.dtype == torch.float32 and shift_state.dtype == torch.float32 and rule_state.stride(0) == shift_state.stride(0)
+        d = TimeMixSpec()
+        d.w_r, d.w_k, d.w_v, d.w_g, d.w_1, d.w_2, d.w_out = self._held(m.w_r, m.w_k, m.w_v, m.w_g, m.w_1, m.w_2, m.w_out)
+        d.mu, d.w0, d.bonus, d.gain = self._held(m.mu, m.w0, m.bonus, m.gain)
+        d.shift_state, d.rule_state, d.slot_stride = shift_state.data_ptr(), rule_state.data_ptr(), int(rule_state.stride(0))
+        self.keep += [shift_state, rule_state]
+        d.heads, d.dim, d.rank, d.eps = m.heads, m.dim, m.rank, m.norm_eps
+        return self._made(L.library().gibbs_plan_body_time_mix(self.handle, ctypes.byref(d)))
 
     def host_body(self, forward: Callable, group: Optional[int] = None) -> int:
         """A mixer or feed-forward written with tensor operations: `forward(h, batch) -> delta [N, hidden]`
@@ -236,6 +304,15 @@ class NativePlan:
         """x += delta (it stays pending until the next norm reads x, which adds it on the way)."""
         self._made(L.library().gibbs_plan_op_add(self.handle, value))
 
+    def normed_delta(self, norm: int, value: int) -> int:
+        """-> value: norm(a body's delta), before it is added; the stream is not touched."""
+        return self._made(L.library().gibbs_plan_op_norm_delta(self.handle, norm, value))
+
+    def reinject(self) -> None:
+        """x += the embedding's output (the rows as the step's first operation saw them)."""
+        self._made(L.library().gibbs_plan_op_reinject(self.handle))
+        self.plain_embedding = False
+
     def drop(self, value: int) -> None:
         self._made(L.library().gibbs_plan_op_drop(self.handle, value))
 
@@ -249,7 +326,11 @@ class NativePlan:
     def build(cls, model, views, rt) -> "NativePlan":
         """The plan of a bound `DecoderModel` (`views[run]`: the cache views of the run's mixers by role)."""
         plan = cls(rt, model.spec.hidden, model.spec.vocab, model.table, model.head, model.head_packed)
+        if model.spec.embedding_scale != 1.0 or model.embedding_inv_freq is not None:
+            plan.embedding(model.spec.embedding_scale, model.embedding_inv_freq)
         for run, i in enumerate(model.spec.order):
+            if run in model.spec.reinject_before:
+                plan.reinject()
             model.blocks[i].emit(plan, views[run])
         plan.tail(model.final_norm.emit(plan))
         return plan

@@ -56,7 +56,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time (each rounded up to whole pages)")
     ap.add_argument("--page-size", type=int, default=None, help="tokens per cache page (default: the engine's)")
-    ap.add_argument("--max-requests", type=int, default=8, help="state slots (live requests)")
+    ap.add_argument("--max-requests", type=int, default=4, help="state slots (live requests)")
     args = ap.parse_args(argv)
 
     print("trace_run: loading kernels and model", file=sys.stderr, flush=True)
