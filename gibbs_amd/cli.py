@@ -112,7 +112,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         cfg = config_from_dict(read_config_json(args.model), tensors=table, arch=args.arch)
         decls = {d.name for d in DecoderModel(cfg.model_spec()).tensor_decls()}
         print(json.dumps({"architecture": cfg.architecture, "config": cfg.to_dict(),
-                          "derived": {"intermediate_size": cfg.intermediate_size, "full_attn_idxs": list(cfg.full_attn_idxs)},
+                          "derived": cfg.derived(),
                           "tensors": {n: list(s) for n, s in sorted(table.items())},
                           "unconsumed": sorted(set(table) - decls), "missing": sorted(decls - set(table))}, indent=1))
         return 0

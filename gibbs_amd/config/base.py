@@ -59,6 +59,10 @@ class ArchConfig:
     def model_spec(self) -> ModelSpec:
         raise NotImplementedError
 
+    def derived(self) -> dict:
+        """Sizes that follow from the configuration's keys by a rule of the architecture (what `--arch-dump` shows)."""
+        return {}
+
 
 def read_config_json(model_dir: str) -> dict:
     path = os.path.join(model_dir, "config.json")

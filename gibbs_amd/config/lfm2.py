@@ -67,6 +67,9 @@ class Lfm2Config(ArchConfig):
     def full_attn_idxs(self) -> Tuple[int, ...]:
         return tuple(i for i, t in enumerate(self.layer_types) if t == ATTENTION)
 
+    def derived(self) -> dict:
+        return {"intermediate_size": self.intermediate_size, "full_attn_idxs": list(self.full_attn_idxs)}
+
     # ------------------------------------------------------------------ reading
     @classmethod
     def from_dict(cls, cfg: Mapping[str, Any],

@@ -114,6 +114,10 @@ class ZokepelConfig(ArchConfig):
     def to_dict(self) -> dict:
         return copy.deepcopy(self.cfg)
 
+    def derived(self) -> dict:
+        order, again = self.run_order()
+        return {"order": list(order), "embedding_added_again_before_runs": list(again)}
+
     # ------------------------------------------------------------------ the model it describes
     def run_order(self) -> Tuple[Tuple[int, ...], Tuple[int, ...]]:
         """(the layers in the order they run, the runs right before which the embedding's output is added again)."""

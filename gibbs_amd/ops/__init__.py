@@ -484,23 +484,100 @@ def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
 def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
                     scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                    slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    slopes: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal grouped-query attention of every row over its request's cache pages.
-    q: [N, >= nh*hd] (row stride free); pages: [num_pages, nkv, page_size, hd]; table: [R, max_pages].
-    `slopes` (float32 [nh]): the score of key k for a query at position p gets slopes[h] * (k - p) added."""
-    require_cuda(q, kpages, vpages, table, pos, row_req, slopes)
+    q: [N, >= nh*hd] (row stride free); key pages: [num_pages, nkv, page_size, hd]; value pages the same with a
+    head size of their own; table: [R, max_pages].
+    `slopes` (float32 [nh]): the score of key k for a query at position p gets slopes[h] * (k - p) added.
+    `bias` (float32 [distances, nh]): it gets bias[min(p - k, distances - 1), h] added."""
+    require_cuda(q, kpages, vpages, table, pos, row_req, slopes, bias)
     assert slopes is None or (slopes.dtype == torch.float32 and slopes.shape == (nh,) and slopes.is_contiguous())
+    assert bias is None or (bias.dtype == torch.float32 and bias.dim() == 2 and bias.shape[1] == nh and bias.is_contiguous())
     assert q.dim() == 2 and q.shape[0] == n_rows and q.stride(1) == 1 and q.shape[1] >= nh * hd
     num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
-    assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
+    vd = vpages.shape[-1]
+    assert _check_pages(vpages, nkv, vd, q.dtype) == (num_pages, page_size)
     assert table.dim() == 2 and table.shape[0] >= n_req
     _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
     if out is None:
-        out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
-    assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
-    call("gibbs_attention_plain", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
-         ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
-         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), ptr(slopes), stream())
+        out = torch.empty((n_rows, nh * vd), dtype=q.dtype, device=q.device)
+    assert out.shape == (n_rows, nh * vd) and out.dtype == q.dtype and out.is_contiguous()
+    call("gibbs_attention_plain_general", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
+         ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd, vd,
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * vd, float(scale), int(window or 0), ptr(slopes), ptr(bias),
+         0 if bias is None else bias.shape[0], stream())
+    return out
+
+
+def qk_unit_kv(rows: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, *, kpages: Optional[torch.Tensor],
+               vpages: Optional[torch.Tensor], table: Optional[torch.Tensor], pos: torch.Tensor, row_req: torch.Tensor,
+               eps: float, unit: bool = True, temp_coef: float = 0.0, temp_every: int = 0) -> None:
+    """rows [N, nh*hd + nkv*hd + nkv*vd], in place: every head of q and k divided by its root mean square
+    (`unit`), q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1), k and v written to their pages."""
+    require_cuda(rows, kpages, vpages, table, pos, row_req)
+    n = rows.shape[0]
+    assert rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] == (nh + nkv) * hd + nkv * vd
+    _i32(pos, n, "pos"); _i32(row_req, n, "row_req")
+    num_pages = page_size = width = 0
+    if kpages is not None:
+        num_pages, page_size = _check_pages(kpages, nkv, hd, rows.dtype)
+        assert _check_pages(vpages, nkv, vd, rows.dtype) == (num_pages, page_size) and table.dtype == torch.int32 and table.is_contiguous()
+        width = table.shape[1]
+    call("gibbs_qk_unit_kv", ptr(rows), rows.shape[1], ptr(kpages), ptr(vpages), dtype_code(rows.dtype), ptr(pos), ptr(row_req),
+         ptr(table), width, page_size, num_pages, n, nh, nkv, hd, vd, float(eps), int(unit), float(temp_coef), int(temp_every), stream())
+
+
+def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor, cu: torch.Tensor,
+                     slot: torch.Tensor, update_state: bool = True) -> torch.Tensor:
+    """float32 [N, C] = silu of a short causal convolution per channel of the ragged rows x [N, C] (taps [C, K], the
+    last one the current token's); `state` [slots, K - 1, C] float32 holds every request's last inputs."""
+    require_cuda(x, taps, state, row_req, cu, slot)
+    n, c = x.shape
+    k = taps.shape[1]
+    assert x.is_contiguous() and taps.dtype == torch.float32 and taps.shape == (c, k) and taps.is_contiguous()
+    assert state.dtype == torch.float32 and state.stride(-1) == 1 and (k == 1 or state.shape[1:] == (k - 1, c))
+    n_req = cu.numel() - 1
+    _i32(row_req, n, "row_req"); _i32(cu, n_req + 1, "cu"); _i32(slot, n_req, "slot")
+    out = torch.empty((n, c), dtype=torch.float32, device=x.device)
+    call("gibbs_causal_conv_silu", ptr(x), c, dtype_code(x.dtype), ptr(taps), ptr(state), state.stride(0), ptr(row_req), ptr(cu),
+         ptr(slot), ptr(out), n, n_req, c, k, int(update_state), stream())
+    return out
+
+
+def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+               cu: torch.Tensor, slot: torch.Tensor, heads: int, kv_heads: int) -> torch.Tensor:
+    """The gated delta rule over ragged rows, all float32: q, k [N, kv_heads*D] (unit vectors, q scaled), v [N, heads*V],
+    beta [N, heads], decay [N, heads] or [N, heads*D]; state [slots, heads, D, V] is read and written.  -> [N, heads*V]."""
+    require_cuda(q, k, v, beta, decay, state, cu, slot)
+    n = q.shape[0]
+    d, vd = q.shape[1] // kv_heads, v.shape[1] // heads
+    for t in (q, k, v, beta, decay):
+        assert t.dtype == torch.float32 and t.is_contiguous() and t.shape[0] == n
+    assert state.dtype == torch.float32 and state.shape[1:] == (heads, d, vd) and state.stride(-1) == 1
+    assert decay.shape[1] in (heads, heads * d) and beta.shape[1] == heads
+    n_req = cu.numel() - 1
+    _i32(cu, n_req + 1, "cu"); _i32(slot, n_req, "slot")
+    out = torch.empty((n, heads * vd), dtype=torch.float32, device=q.device)
+    call("gibbs_delta_rule", ptr(q), ptr(k), q.shape[1], ptr(v), v.shape[1], ptr(beta), ptr(decay), int(decay.shape[1] != heads),
+         ptr(state), state.stride(0), ptr(cu), ptr(slot), ptr(out), n_req, heads, kv_heads, d, vd, stream())
+    return out
+
+
+def decayed_outer_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor, bonus: torch.Tensor, state: torch.Tensor,
+                       cu: torch.Tensor, slot: torch.Tensor, heads: int) -> torch.Tensor:
+    """o_t = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T, per head over ragged rows: r, k, v [N, heads*D] in
+    one type, w float32 [N, heads*D], bonus float32 [heads, D]; state [slots, heads, D, D] float32.  -> float32 [N, heads*D]."""
+    require_cuda(r, k, v, w, bonus, state, cu, slot)
+    n, c = r.shape
+    d = c // heads
+    assert k.shape == r.shape == v.shape and k.dtype == r.dtype == v.dtype and all(t.is_contiguous() for t in (r, k, v, w, bonus))
+    assert w.dtype == torch.float32 and w.shape == (n, c) and bonus.dtype == torch.float32 and bonus.shape == (heads, d)
+    assert state.dtype == torch.float32 and state.shape[1:] == (heads, d, d) and state.stride(-1) == 1
+    n_req = cu.numel() - 1
+    _i32(cu, n_req + 1, "cu"); _i32(slot, n_req, "slot")
+    out = torch.empty((n, c), dtype=torch.float32, device=r.device)
+    call("gibbs_decayed_outer_rule", ptr(r), ptr(k), ptr(v), dtype_code(r.dtype), ptr(w), ptr(bonus), ptr(state), state.stride(0),
+         ptr(cu), ptr(slot), ptr(out), n_req, heads, d, stream())
     return out
 
 

@@ -54,6 +54,17 @@ _SIGNATURES = {
                          c_void_p],
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p, c_void_p],
+    "gibbs_attention_plain_general": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                      c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p,
+                                      c_void_p, c_int, c_void_p],
+    "gibbs_qk_unit_kv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int, c_void_p],
+    "gibbs_causal_conv_silu": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                               c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_delta_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p,
+                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_decayed_outer_rule": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_int, c_int, c_void_p],
     "gibbs_decode_tail": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,

@@ -142,8 +142,9 @@ def biased_attention(h, w, p, eps: float) -> np.ndarray:
     k = unit_rms((h @ w["k"].T).reshape(T, G, D), eps)
     v = (h @ w["v"].T).reshape(T, G, V)
     pos = np.arange(T)
-    temp = 1.0 + p["q_temp"]["coef"] * np.log(np.floor((pos + 1) / p["q_temp"]["every"]) + 1.0)
-    q = q * temp[:, None, None]
+    if p.get("q_temp") is not None:                     # a temperature on the queries that grows with the position
+        temp = 1.0 + p["q_temp"]["coef"] * np.log(np.floor((pos + 1) / p["q_temp"]["every"]) + 1.0)
+        q = q * temp[:, None, None]
     rel = w["rel"]
     buckets = np.array([distance_bucket(n, rel.shape[0], p["bias_max"]) for n in range(T)], dtype=np.int64)
     dist = pos[:, None] - pos[None, :]
