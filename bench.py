@@ -277,8 +277,87 @@ def parity(layers: int = 3) -> dict:
             "bf16_loop_tokens_are_stepped": loop_tokens["bfloat16"] == step_tokens["bfloat16"], "pass": bool(ok)}
 
 
+# ----------------------------------------------------------------------------------------------- another design beside the headline
+def zokepel_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Zokepel model of `layers` layers (parallel, channel_delta, delta in turn) whose sizes resemble a real
+    model's at this width: heads of 64 for the attention and the time mixing, heads of 128 for the delta rules."""
+    heads64, heads128 = width // 64, width // 128
+    left = {"heads": heads64, "kv_heads": max(1, heads64 // 4), "dim": 64, "vdim": 64, "bias_rows": 32, "bias_max": 4096,
+            "scale": 0.125, "q_temp": {"coef": 0.1, "every": 1024}}
+    kinds = [
+        {"type": "parallel", "mixer": {"left": left, "right": {"heads": heads64, "dim": 64, "decay_rank": 64}}},
+        {"type": "channel_delta", "mixer": {"heads": heads128, "kv_heads": heads128, "dim": 128, "vdim": 128, "conv": 4,
+                                            "decay_rank": 64, "gate_rank": 64}},
+        {"type": "delta", "mixer": {"heads": heads128, "kv_heads": max(1, heads128 // 2), "dim": 128, "vdim": 128, "conv": 4}},
+    ]
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    return {"architecture": "Zokepel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "layers": [dict(kinds[i % 3], mlp=mlp) for i in range(layers)]}
+
+
+def lfm2_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """The closest model the framework had: LFM2 at the same width, feed-forward, depth and vocabulary, a third of
+    its layers attention (where the other design has its attention)."""
+    return dict(SHAPE, hidden_size=width, num_hidden_layers=layers, full_attn_idxs=[i for i in range(layers) if i % 3 == 0],
+                num_attention_heads=width // 64, num_key_value_heads=max(1, width // 256), block_ff_dim=ff,
+                block_auto_adjust_ff_dim=False, vocab_size=vocab, tie_embedding=False)
+
+
+def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
+    import torch
+
+    from gibbs_amd import Engine
+    from gibbs_amd.config import config_from_dict
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import random_weights_on_device
+    cfg = config_from_dict(shape)
+    decls = DecoderModel(cfg.model_spec()).tensor_decls()
+    compute = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0", bias_std=0.5)
+    return Engine(config=cfg, weights=weights, dtype=dtype, max_tokens=max_requests * context, max_requests=max_requests, ctx=context)
+
+
+def compare_designs(args) -> int:
+    """`--design zokepel`: prefill and decode speed of Zokepel at a few sizes beside LFM2 at equal width, depth,
+    feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One JSON line."""
+    import gc
+
+    import torch
+
+    from gibbs_amd import roofline as R
+    sizes = {"small": [(1024, 4096, 6, 32768)], "medium": [(2048, 8192, 6, 65536)],
+             "all": [(1024, 4096, 6, 32768), (2048, 8192, 6, 65536), (4096, 12288, 3, 65536)]}[args.sizes]
+    rows = []
+    for width, ff, layers, vocab in sizes:
+        for design, shape in (("Zokepel", zokepel_shape(width, ff, layers, vocab)), ("LFM2", lfm2_shape(width, ff, layers, vocab))):
+            engine = engine_of(shape, args.dtype, max_requests=args.batch, context=4096)
+            row = {"design": design, "width": width, "ff": ff, "layers": layers, "vocab": vocab}
+            prefill_s = time_prefill(engine, n_tokens=args.prefill_tokens)
+            row["prefill_tok_s"] = round(args.prefill_tokens / prefill_s, 1)
+            row["prefill_ms"] = round(prefill_s * 1e3, 3)
+            row["prefill_frac_of_peak"] = round(R.prefill_flops(engine, args.prefill_tokens) / prefill_s / R.PEAK_FLOPS[args.dtype], 4)
+            if not args.no_kernels:
+                ids = seeded_prompt(5, args.prefill_tokens, vocab)
+                row["prefill_kernels"] = kernel_shares(lambda: (engine.step([("k", ids, [len(ids) - 1])]), engine.release("k")), most=10)
+            dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels, prompt_len=args.prompt_len)
+            row["decode_tok_s"] = round(args.batch * args.steps / dt, 1)
+            row["decode_ms_per_step"] = round(dt / args.steps * 1e3, 4)
+            row["decode_frac_of_hbm"] = round(R.decode_bytes(engine, seq_lens) / (dt / args.steps) / R.HBM_BYTES_PER_S, 4)
+            row["decode_kernels"] = top
+            rows.append(row)
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": f"prefill and decode tok/s of two designs at equal sizes (batch {args.batch}, {args.prompt_len}-token prompts)",
+                      "dtype": args.dtype, "data": "synthetic", "steps": args.steps, "warmup": args.warmup, "rows": rows}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=["lfm2", "zokepel"], default="lfm2",
+                    help="zokepel: that design beside LFM2 at equal sizes instead of the headline workload")
+    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -306,6 +385,8 @@ def main() -> int:
         print(f"--prompt-len + --warmup + {RUNS + 1} x --steps must stay below the context ({context})")
         return 2
 
+    if args.design == "zokepel":
+        return compare_designs(args)
     from gibbs_amd import roofline as R
     gate = None if args.no_parity else parity()
     engine = build_engine(args.dtype, args.layers, max_requests=args.batch if args.no_points else max(64, args.batch),

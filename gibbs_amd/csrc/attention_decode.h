@@ -167,6 +167,10 @@ struct DecodeArgs {
   // of the first keys).  A row that is beyond the bound after all takes the ids of its slice as it would without.
   int ids_whole, n_ids;
   int merge_here;   // the last slice of a (row, group of heads) to finish merges them (else a second kernel does)
+  // a bias on the scores by distance, or null (the matrix-core walk only): [nh, bias_len], row h entry d for keys d
+  // positions back (the last entry for all farther ones), divided by `scale` already
+  const float* bias;
+  int bias_len;
 };
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -442,6 +446,13 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
             s4[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qb[s2], s4[c], 0, 0, 0);
           }
         }
+        if (a.bias) {
+          const float* bias = a.bias + (size_t)(kvh * G + g0 + min(lr, gcount - 1)) * a.bias_len;
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s4[c][i] += bias[min(max(p - (t0 + c * 16 + g4 * 4 + i), 0), a.bias_len - 1)];
+        }
         // keys beyond the slice (the last tile); maximum of the raw scores (the scale is positive)
         float mx = -INFINITY;
 #pragma unroll
@@ -668,6 +679,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   const long longest = (bound + a.n_splits - 1) / a.n_splits + 8 * TILE;
   const bool mm_can = a.hd % 16 == 0 && a.hd <= 128 && longest / a.page_size + 2 <= SEG_PAGES;
   GIBBS_REQUIRE(kind != 2 || mm_can, "attention_decode: the matrix-core kernel takes head sizes in steps of 16 up to 128 and key slices of at most %d pages (head size %d, %ld keys a slice)", SEG_PAGES - 2, a.hd, longest);
+  GIBBS_REQUIRE(!a.bias || (mm_can && kind != 1), "attention_decode: a bias on the scores takes the matrix-core kernel (head sizes in steps of 16 up to 128)");
   const bool mm = kind == 2 || (kind == 0 && mm_can);
   const long ids = (bound + a.page_size - 1) / a.page_size;
   a.ids_whole = a.window == 0 && ids <= SEG_PAGES;

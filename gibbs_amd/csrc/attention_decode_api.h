@@ -34,6 +34,13 @@ int gibbs_attention_decode_static(const void* q, const void* kpages, const void*
                                   int num_pages, int n_rows, int nh, int nkv, int hd, long ldq, long ldo, float scale,
                                   int window, int n_splits, int waves, int kind, int max_keys, hipStream_t stream);
 
+// gibbs_attention_decode with a bias on the scores by distance: float32 [nh, bias_len], the score of a key d positions
+// back gets bias[h][min(d, bias_len - 1)] * scale added (null: none).  The matrix-core walk only.
+int gibbs_attention_decode_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial, const int* pos,
+                                const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
+                                int nh, int nkv, int hd, long ldq, long ldo, float scale, int window, int n_splits, int waves,
+                                int kind, int max_keys, const float* bias, int bias_len, hipStream_t stream);
+
 // Floats of the per-GPU array behind gibbs_attention_decode_static (2 Mi floats = 8 MiB).
 long gibbs_attention_decode_static_capacity(void);
 

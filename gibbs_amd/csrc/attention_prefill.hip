@@ -69,6 +69,10 @@ struct PrefillArgs {
   float scale;
   int window;
   int n_splits;    // slices of the key tiles (1: the workgroup writes the finished rows)
+  // a bias on the scores by distance, or null: [nh, bias_len], row h entry d for keys d positions back (the last
+  // entry for all farther ones), divided by `scale` already (it is added to the raw scores, which are scaled later)
+  const float* bias;
+  int bias_len;
 };
 
 // DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
@@ -238,6 +242,16 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
   auto weights = [&](floatx4 (&s4)[4], int key0, bf16x8 (&pf)[2]) {
     // mask by position (only the tiles on the rows' diagonal, or with a window: the same for the whole wave,
     // and said so, or the selects are done for every tile), row maximum (of the raw scores: the scale is positive)
+    if (a.bias) {
+      const float* bias = a.bias + (size_t)head * a.bias_len;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int back = pos_row - (key0 + c * 16 + g * 4 + i);     // (keys ahead of the row are masked below)
+          s4[c][i] += bias[min(max(back, 0), a.bias_len - 1)];
+        }
+    }
     const bool need_mask = __builtin_amdgcn_readfirstlane((int)(key0 + BN - 1 > p0 + wave * 16 || a.window > 0)) != 0;
     if (need_mask) {
 #pragma unroll
@@ -416,11 +430,13 @@ void launch_prefill(dim3 grid, int heads_per_wg, hipStream_t stream, const bf16*
 // of a step from some request on): first_row = cu[0] then, and n_rows counts the rows from there.
 // heads_per_wg: query heads of a kv head's group that a workgroup takes (1, 2 or 4; 0 counts as 1; the step's
 // rule for it is gibbs_rule_prefill_heads).
-GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
-                                         const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
-                                         int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                         long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
-                                         hipStream_t stream) {
+// bias (or null): float32 [nh, bias_len], the score of a key d positions back gets bias[h][min(d, bias_len - 1)] * scale added.
+GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                              const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
+                                              int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                              long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
+                                              const float* bias, int bias_len, hipStream_t stream) {
+  GIBBS_REQUIRE(!bias || (bias_len > 0 && scale > 0.f), "attention_prefill: an empty table of score biases, or a scale that is not positive");
   GIBBS_REQUIRE(n_rows >= 0 && n_req >= 0 && nh > 0 && nkv > 0, "attention_prefill: bad sizes rows=%d requests=%d heads=%d kv=%d", n_rows, n_req, nh, nkv);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 128, "attention_prefill: head size %d must be a multiple of 16 up to 128", hd);
@@ -434,7 +450,7 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
                 "attention_prefill: %d heads a workgroup (1, 2 or 4 of a kv head's %d; more than one for head sizes up to 64)", heads_per_wg, nh / nkv);
   if (n_rows == 0 || n_req == 0) return 0;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits};
+  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits, bias, bias_len};
   dim3 grid(ceil_div(n_rows, BM) + n_req, nh, n_splits);
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;
@@ -456,4 +472,13 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
                            nh, hd, n_splits, ldo);
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
+}
+
+GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                         const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
+                                         int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                         long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
+                                         hipStream_t stream) {
+  return gibbs_attention_prefill_bias(q, kpages, vpages, out, partial, cu, ctx, table, n_req, max_pages, page_size, num_pages, n_rows,
+                                      nh, nkv, hd, ldq, ldo, scale, window, n_splits, first_row, heads_per_wg, nullptr, 0, stream);
 }

@@ -126,15 +126,21 @@ struct RecurrenceArgs {
   int H, G, D, V;
 };
 
-// One wave per (request, head, 16 columns of the state).  A column of S [D, V] is spread over 4 lanes (key
-// channel i belongs to lane part i % 4, so a lane holds DPT = ceil(D / 4) values in registers); sums over the
-// key channels are folded over those 4 lanes.  The operands of 8 tokens at a time go through LDS.
+// One wave per (request, head, COLS columns of the state).  A column of S [D, V] is spread over PARTS lanes (lane
+// part p holds the DPT key channels p DPT .. p DPT + DPT - 1 in registers; COLS = 64 / PARTS), so that a head
+// gives many short waves instead of a few long ones: the walk over a request's tokens is a chain in which every
+// token waits for the one before, and what fills the chip is the number of independent chains.  Sums over the
+// key channels are folded over the PARTS lanes.  The operands of 8 tokens at a time go through LDS; the next 8
+// are on their way from memory into registers meanwhile.
 //   delta:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //   outer:  o = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T
-template <typename TIn, int RULE, int DPT>
+template <typename TIn, int RULE, int DPT, int PARTS>
 __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
-  constexpr int PARTS = 4, COLS = 16, TOK = 8, DMAX = DPT * PARTS;
-  __shared__ float sq[TOK][DMAX], sk[TOK][DMAX], sd[TOK][DMAX], sv[TOK][COLS], sb[TOK], sg[TOK];
+  constexpr int COLS = WAVE / PARTS, TOK = 8, DMAX = DPT * PARTS, LDP = DPT + 4, PER_LANE = TOK * DMAX / WAVE;
+  constexpr int V_PER_LANE = (TOK * COLS + WAVE - 1) / WAVE;
+  static_assert(DPT % 4 == 0 && TOK * DMAX % WAVE == 0, "a lane reads its channels four at a time");
+  __shared__ __attribute__((aligned(16))) float sq[TOK][PARTS][LDP], sk[TOK][PARTS][LDP], sd[TOK][PARTS][LDP];
+  __shared__ float sv[TOK][COLS], sb[TOK], sg[TOK];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int col = lane / PARTS, part = lane % PARTS;
   const int j = blockIdx.z * COLS + col;
@@ -145,7 +151,7 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
   float S[DPT], bonus[DPT];
 #pragma unroll
   for (int ii = 0; ii < DPT; ++ii) {
-    const int i = ii * PARTS + part;
+    const int i = part * DPT + ii;
     S[ii] = (i < D && j < V) ? st[(size_t)i * V + j] : 0.f;
     bonus[ii] = (RULE == RULE_OUTER && i < D) ? a.bonus[(size_t)h * D + i] : 0.f;
   }
@@ -153,79 +159,122 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
   const TIn* k = (const TIn*)a.k;
   const TIn* v = (const TIn*)a.v;
   const bool channel_decay = RULE == RULE_OUTER || a.per_channel;
-  for (int t0 = 0; t0 < rows; t0 += TOK) {
+  // the next 8 tokens' operands, in registers until the current 8 are done with LDS
+  float rq[PER_LANE], rk[PER_LANE], rd[PER_LANE], rv[V_PER_LANE], rb = 0.f, rg = 1.f;
+  auto ask = [&](int t0) {
     const int nt = min(TOK, rows - t0);
-    __syncthreads();
-    for (int idx = lane; idx < TOK * DMAX; idx += WAVE) {
-      const int t = idx / DMAX, i = idx % DMAX;
+#pragma unroll
+    for (int e = 0; e < PER_LANE; ++e) {
+      const int idx = e * WAVE + lane, t = idx / DMAX, i = idx % DMAX;
       const bool live = t < nt && i < D;
       const size_t row = (size_t)(first + t0 + (t < nt ? t : 0));
-      sq[t][i] = live ? to_float(q[row * a.ldq + (size_t)kvh * D + i]) : 0.f;
-      sk[t][i] = live ? to_float(k[row * a.ldk + (size_t)kvh * D + i]) : 0.f;
-      if (channel_decay) sd[t][i] = live ? a.decay[row * a.H * D + (size_t)h * D + i] : 1.f;
+      const int ic = i < D ? i : 0;
+      rq[e] = live ? to_float(q[row * a.ldq + (size_t)kvh * D + ic]) : 0.f;
+      rk[e] = live ? to_float(k[row * a.ldk + (size_t)kvh * D + ic]) : 0.f;
+      rd[e] = (channel_decay && live) ? a.decay[row * a.H * D + (size_t)h * D + ic] : 1.f;
     }
-    for (int idx = lane; idx < TOK * COLS; idx += WAVE) {
-      const int t = idx / COLS, c = idx % COLS, jj = blockIdx.z * COLS + c;
-      sv[t][c] = (t < nt && jj < V) ? to_float(v[(size_t)(first + t0 + t) * a.ldv + (size_t)h * V + jj]) : 0.f;
+#pragma unroll
+    for (int e = 0; e < V_PER_LANE; ++e) {
+      const int idx = e * WAVE + lane, t = idx / COLS, jj = blockIdx.z * COLS + idx % COLS;
+      rv[e] = (t < nt && jj < V) ? to_float(v[(size_t)(first + t0 + t) * a.ldv + (size_t)h * V + jj]) : 0.f;
     }
     if (RULE == RULE_DELTA && lane < TOK) {
       const bool live = lane < nt;
       const size_t row = (size_t)(first + t0 + (live ? lane : 0));
-      sb[lane] = live ? a.beta[row * a.H + h] : 0.f;
-      sg[lane] = (live && !a.per_channel) ? a.decay[row * a.H + h] : 1.f;
+      rb = live ? a.beta[row * a.H + h] : 0.f;
+      rg = (live && !a.per_channel) ? a.decay[row * a.H + h] : 1.f;
     }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int e = 0; e < PER_LANE; ++e) {
+      const int idx = e * WAVE + lane, t = idx / DMAX, i = idx % DMAX;
+      sq[t][i / DPT][i % DPT] = rq[e];
+      sk[t][i / DPT][i % DPT] = rk[e];
+      sd[t][i / DPT][i % DPT] = rd[e];
+    }
+#pragma unroll
+    for (int e = 0; e < V_PER_LANE; ++e) {
+      const int idx = e * WAVE + lane;
+      if (idx < TOK * COLS) sv[idx / COLS][idx % COLS] = rv[e];
+    }
+    if (RULE == RULE_DELTA && lane < TOK) {
+      sb[lane] = rb;
+      sg[lane] = rg;
+    }
+  };
+  auto fold = [&](float x) {
+#pragma unroll
+    for (int o = 1; o < PARTS; o <<= 1) x += __shfl_xor(x, o, WAVE);
+    return x;
+  };
+  if (rows > 0) ask(0);
+  for (int t0 = 0; t0 < rows; t0 += TOK) {
+    const int nt = min(TOK, rows - t0);
+    __syncthreads();   // everyone is done with the tokens before
+    put();
     __syncthreads();
+    if (t0 + TOK < rows) ask(t0 + TOK);
     for (int t = 0; t < nt; ++t) {
       const float vj = sv[t][col];
-      float o = 0.f;
+      float kk[DPT], qq[DPT], dd[DPT];
+#pragma unroll
+      for (int c = 0; c < DPT / 4; ++c) {
+        const float4 k4 = *(const float4*)&sk[t][part][c * 4], q4 = *(const float4*)&sq[t][part][c * 4];
+        kk[c * 4] = k4.x; kk[c * 4 + 1] = k4.y; kk[c * 4 + 2] = k4.z; kk[c * 4 + 3] = k4.w;
+        qq[c * 4] = q4.x; qq[c * 4 + 1] = q4.y; qq[c * 4 + 2] = q4.z; qq[c * 4 + 3] = q4.w;
+        if (channel_decay) {
+          const float4 d4 = *(const float4*)&sd[t][part][c * 4];
+          dd[c * 4] = d4.x; dd[c * 4 + 1] = d4.y; dd[c * 4 + 2] = d4.z; dd[c * 4 + 3] = d4.w;
+        }
+      }
+      float o0 = 0.f, o1 = 0.f;
       if (RULE == RULE_DELTA) {
         const float g_head = sg[t];
-        float dot = 0.f;
+        float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
-        for (int ii = 0; ii < DPT; ++ii) {
-          const int i = ii * PARTS + part;
-          const float s = S[ii] * (channel_decay ? sd[t][i] : g_head);
-          S[ii] = s;
-          dot = fmaf(s, sk[t][i], dot);
+        for (int ii = 0; ii < DPT; ii += 2) {
+          S[ii] *= channel_decay ? dd[ii] : g_head;
+          S[ii + 1] *= channel_decay ? dd[ii + 1] : g_head;
+          dot0 = fmaf(S[ii], kk[ii], dot0);
+          dot1 = fmaf(S[ii + 1], kk[ii + 1], dot1);
         }
-        dot += __shfl_xor(dot, 1, WAVE);
-        dot += __shfl_xor(dot, 2, WAVE);
-        const float u = sb[t] * (vj - dot);
+        const float u = sb[t] * (vj - fold(dot0 + dot1));
 #pragma unroll
-        for (int ii = 0; ii < DPT; ++ii) {
-          const int i = ii * PARTS + part;
-          const float s = fmaf(sk[t][i], u, S[ii]);
-          S[ii] = s;
-          o = fmaf(s, sq[t][i], o);
+        for (int ii = 0; ii < DPT; ii += 2) {
+          S[ii] = fmaf(kk[ii], u, S[ii]);
+          S[ii + 1] = fmaf(kk[ii + 1], u, S[ii + 1]);
+          o0 = fmaf(S[ii], qq[ii], o0);
+          o1 = fmaf(S[ii + 1], qq[ii + 1], o1);
         }
       } else {
 #pragma unroll
-        for (int ii = 0; ii < DPT; ++ii) {
-          const int i = ii * PARTS + part;
-          const float kv = sk[t][i] * vj;
-          o = fmaf(sq[t][i], fmaf(bonus[ii], kv, S[ii]), o);
-          S[ii] = fmaf(sd[t][i], S[ii], kv);
+        for (int ii = 0; ii < DPT; ii += 2) {
+          const float kv0 = kk[ii] * vj, kv1 = kk[ii + 1] * vj;
+          o0 = fmaf(qq[ii], fmaf(bonus[ii], kv0, S[ii]), o0);
+          o1 = fmaf(qq[ii + 1], fmaf(bonus[ii + 1], kv1, S[ii + 1]), o1);
+          S[ii] = fmaf(dd[ii], S[ii], kv0);
+          S[ii + 1] = fmaf(dd[ii + 1], S[ii + 1], kv1);
         }
       }
-      o += __shfl_xor(o, 1, WAVE);
-      o += __shfl_xor(o, 2, WAVE);
+      const float o = fold(o0 + o1);
       if (part == 0 && j < V) a.out[(size_t)(first + t0 + t) * a.H * V + (size_t)h * V + j] = o;
     }
   }
 #pragma unroll
   for (int ii = 0; ii < DPT; ++ii) {
-    const int i = ii * PARTS + part;
+    const int i = part * DPT + ii;
     if (i < D && j < V) st[(size_t)i * V + j] = S[ii];
   }
 }
 
+// Lanes per column by the key size: 8 channels a lane up to 128 channels, 16 beyond.
 template <typename TIn, int RULE>
 int launch_recurrence(const RecurrenceArgs& a, int n_req, hipStream_t stream) {
-  const dim3 grid(n_req, a.H, ceil_div(a.V, 16));
-  if (a.D <= 32) recurrence_kernel<TIn, RULE, 8><<<grid, 64, 0, stream>>>(a);
-  else if (a.D <= 64) recurrence_kernel<TIn, RULE, 16><<<grid, 64, 0, stream>>>(a);
-  else if (a.D <= 128) recurrence_kernel<TIn, RULE, 32><<<grid, 64, 0, stream>>>(a);
-  else recurrence_kernel<TIn, RULE, 64><<<grid, 64, 0, stream>>>(a);
+  if (a.D <= 32) recurrence_kernel<TIn, RULE, 8, 4><<<dim3(n_req, a.H, ceil_div(a.V, 16)), 64, 0, stream>>>(a);
+  else if (a.D <= 64) recurrence_kernel<TIn, RULE, 8, 8><<<dim3(n_req, a.H, ceil_div(a.V, 8)), 64, 0, stream>>>(a);
+  else if (a.D <= 128) recurrence_kernel<TIn, RULE, 8, 16><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
+  else recurrence_kernel<TIn, RULE, 16, 16><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
   return 0;
 }
 

@@ -450,7 +450,8 @@ struct AttnBody : Body {
   int vd = 0;
   int unit_qk = 0, temp_every = 0;
   float temp_coef = 0.f;
-  const float* bias = nullptr;
+  const float* bias = nullptr;        // [bias_len, nh]
+  const float* bias_t = nullptr;      // the same as [nh, bias_len] divided by the scale: what the matrix-core kernels add to raw scores
   int bias_len = 0;
   bool extras() const { return vd != hd || unit_qk || temp_every > 0 || bias; }
   int cache_group() const override { return group; }
@@ -486,8 +487,9 @@ struct AttnBody : Body {
     int n_splits, waves;
     decode_splits(n_rows, nkv, nh / nkv, e.a.max_seq, hd, page_size, 0, &n_splits, &waves);
     float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(n_rows, nh, hd, n_splits) * 4) : nullptr;
-    RUN(e, gibbs_attention_decode(q, kpages, vpages, o, partial, pos, row_req, e.table(group), e.width(group), page_size, num_pages,
-                                  n_rows, nh, nkv, hd, ldq, (long)nh * hd, scale, window, n_splits, waves, 0, e.a.max_seq, e.a.stream));
+    RUN(e, gibbs_attention_decode_bias(q, kpages, vpages, o, partial, pos, row_req, e.table(group), e.width(group), page_size, num_pages,
+                                       n_rows, nh, nkv, hd, ldq, (long)nh * hd, scale, window, n_splits, waves, 0, e.a.max_seq, bias_t,
+                                       bias_len, e.a.stream));
     e.give(partial);
   }
   // q/k norm, rotation and the cache write of the step's rows (a mixer that reads another's cache writes nothing)
@@ -533,8 +535,11 @@ struct AttnBody : Body {
       const int* table = e.table(group);
       const int width = e.width(group);
       att = e.take((long)N * ldo * e.esize);
-      const bool fast_bf16 = e.bf16_run && !slopes && !extras();   // (the fast kernels take no score bias)
-      if (fast_bf16 && a.max_q > 1 && hd % 16 == 0 && hd <= 128) {
+      // the matrix-core kernels take rows that are prepared (whatever prepared them), keys and values of one head
+      // size, and a bias on the scores as a table over the distance (no slopes)
+      const bool matrix_sizes = hd % 16 == 0 && hd <= 128;
+      const bool fast_bf16 = e.bf16_run && !slopes && vd == hd && (!bias || (bias_t && matrix_sizes));
+      if (fast_bf16 && a.max_q > 1 && matrix_sizes) {
         // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
         // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
         // matrix-core kernel
@@ -543,9 +548,9 @@ struct AttnBody : Body {
         const int rows = N - lead, reqs = a.n_req - lead;
         const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), nh, a.max_seq, window) : 1;
         float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(N, nh, hd, n_splits) * 4) : nullptr;
-        RUN(e, gibbs_attention_prefill(raw, kpages, vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
-                                       width, page_size, num_pages, rows, nh, nkv, hd, ldq, ldo, scale, window, n_splits, lead,
-                                       prefill_heads(rows, reqs, nh, nkv, hd, a.max_seq, n_splits), a.stream));
+        RUN(e, gibbs_attention_prefill_bias(raw, kpages, vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
+                                            width, page_size, num_pages, rows, nh, nkv, hd, ldq, ldo, scale, window, n_splits, lead,
+                                            prefill_heads(rows, reqs, nh, nkv, hd, a.max_seq, n_splits), bias_t, bias_len, a.stream));
         e.give(partial);
       } else if (fast_bf16 && a.max_q == 1 && hd % 8 == 0) {
         decode_attention(e, raw, ldq, N, a.pos, a.row_req, att);
@@ -939,7 +944,7 @@ GIBBS_EXPORT int gibbs_plan_embedding(void* plan, float scale, const float* inv_
 }
 
 GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, float temp_coef, int temp_every,
-                                             const float* bias, int bias_len) {
+                                             const float* bias, const float* bias_t, int bias_len) {
   Plan* p = open_plan(plan);
   if (!p) return -1;
   AttnBody* t = p->has_body(body) ? dynamic_cast<AttnBody*>(p->bodies[body].get()) : nullptr;
@@ -948,7 +953,7 @@ GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int u
     gibbs_fail("plan: an attention with these extras has no rotation, no q/k gains, no hook and no slopes, and owns its pages");
     return -1;
   }
-  t->vd = vd; t->unit_qk = unit_qk; t->temp_coef = temp_coef; t->temp_every = temp_every; t->bias = bias; t->bias_len = bias ? bias_len : 0;
+  t->vd = vd; t->unit_qk = unit_qk; t->temp_coef = temp_coef; t->temp_every = temp_every; t->bias = bias; t->bias_t = bias ? bias_t : nullptr; t->bias_len = bias ? bias_len : 0;
   t->qkv.O = (t->nh + t->nkv) * t->hd + t->nkv * vd;
   t->out.I = t->nh * vd;
   return 0;

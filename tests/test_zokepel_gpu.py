@@ -20,8 +20,8 @@ from tests.test_engine_gpu import mixed_schedule, portions, run_steps
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["P", "Q", "R"]
-LENGTHS = {"P": 150, "Q": 210, "R": 120}
+NAMES = ["P", "Q", "R", "S"]
+LENGTHS = {"P": 150, "Q": 210, "R": 120, "S": 330}
 # bfloat16 against the plain implementation, per row: relative L2 error of the logits (1.5 x the worst row measured
 # for these models; a wrong bucket, a lost state or a missing scale shows as tens of percent)
 BF16_REL_L2 = 0.06

@@ -58,7 +58,20 @@ ZOKEPEL_R = {
          "mlp": _mlp(100, 3.0)},
     ],
 }
-MODELS = {"P": ZOKEPEL_P, "Q": ZOKEPEL_Q, "R": ZOKEPEL_R}
+# S: heads of 64 in groups of four with keys and values of one size (in bfloat16 the matrix-core attention kernels, with
+# the distance bias), a table whose reach is shorter than the sequences, delta-rule heads of 128 key channels.
+ZOKEPEL_S = {
+    "architecture": "Zokepel", "vocab": 512, "width": 256, "norm": {"eps": 1e-6}, "embedding": {"scale": 2.0},
+    "layers": [
+        {"type": "parallel", "mixer": {"left": _left(8, 2, 64, 64, 16, 100, 0.125, (0.5, 64)),
+                                       "right": {"heads": 4, "dim": 64, "decay_rank": 32}}, "mlp": _mlp(512, 7.0)},
+        {"type": "delta", "mixer": {"heads": 4, "kv_heads": 2, "dim": 128, "vdim": 64, "conv": 4}, "mlp": _mlp(512, 7.0)},
+        {"type": "parallel", "mixer": {"left": _left(4, 4, 32, 32, 10, 64, 0.2, (0.3, 32)),
+                                       "right": {"heads": 8, "dim": 32, "decay_rank": 8}}, "mlp": None},
+    ],
+    "loop": {"start": 0, "stop": 2, "times": 2},
+}
+MODELS = {"P": ZOKEPEL_P, "Q": ZOKEPEL_Q, "R": ZOKEPEL_R, "S": ZOKEPEL_S}
 
 
 def single_layer(kind: str) -> dict:
