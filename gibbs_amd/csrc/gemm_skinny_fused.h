@@ -56,6 +56,7 @@ struct FusedArgs {
   const int* ctx;   // [N] cached length of each row's request (history rows before position 0 are zero)
   int K;
   int act;  // GLU: the activation's code
+  float act_alpha, act_limit;   // of the clamped variant (ACT_CLAMPED_SWISH)
 };
 
 // KC: the convolution's kernel length when it is 2..4 (its operands are then asked for before the
@@ -467,7 +468,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float gt = sum[0][i] * scale, up = sum[RG > 1 ? 1 : 0][i] * scale;
-        v[i] = (bf16)(activate_to_bf16(gt, a.act) * up);
+        v[i] = (bf16)(a.act == ACT_CLAMPED_SWISH ? clamped_swish_product(gt, up, a.act_alpha, a.act_limit) : activate_to_bf16(gt, a.act) * up);
       }
       if (full && a.y_vec) *(bf16x4*)y = bf16x4{v[0], v[1], v[2], v[3]};
       else for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = v[i];

@@ -75,12 +75,21 @@ GIBBS_EXPORT int gibbs_skinny_residual(const void* X, const void* W, float* x, v
 }
 
 // out[n, f] = silu(s_n gate_f . X_n) * (s_n up_f . X_n); W = [gate rows (F); up rows (F)], rms prologue.
+// act ACT_CLAMPED_SWISH takes alpha and limit (see activation.h); the other codes ignore them.
+GIBBS_EXPORT int gibbs_skinny_glu_general(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw,
+                                          long ldy, int rms, float eps, int act, float alpha, float limit, hipStream_t stream);
 GIBBS_EXPORT int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw,
                                   long ldy, int rms, float eps, int act, hipStream_t stream) {
+  GIBBS_REQUIRE(act >= 0 && act < ACT_COUNT, "skinny_glu: unknown activation %d", act);
+  return gibbs_skinny_glu_general(X, W, Y, N, F, I, ldx, ldw, ldy, rms, eps, act, 0.f, 0.f, stream);
+}
+GIBBS_EXPORT int gibbs_skinny_glu_general(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw,
+                                          long ldy, int rms, float eps, int act, float alpha, float limit, hipStream_t stream) {
   if (check_common("skinny_glu", X, W, N, F, I, ldx, ldw)) return 1;
   GIBBS_REQUIRE(ldy >= F, "skinny_glu: output rows shorter than %d", F);
-  GIBBS_REQUIRE(act >= 0 && act < ACT_COUNT, "skinny_glu: unknown activation %d", act);
+  GIBBS_REQUIRE((act >= 0 && act < ACT_COUNT) || (act == ACT_CLAMPED_SWISH && limit > 0.f), "skinny_glu: unknown activation %d", act);
   FusedArgs a{};
+  a.act_alpha = alpha; a.act_limit = limit;
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy; a.act = act;
   a.y_vec = ldy % 4 == 0 && ((uintptr_t)Y % 8) == 0;

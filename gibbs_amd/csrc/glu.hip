@@ -39,9 +39,7 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ out
   const int n = blockIdx.x;
   const int f = blockIdx.y * blockDim.x + threadIdx.x;
   if (f >= F) return;
-  const float g = fminf(to_float(gu[(size_t)n * 2 * F + f]), limit);
-  const float u = fminf(fmaxf(to_float(gu[(size_t)n * 2 * F + F + f]), -limit), limit);
-  out[(size_t)n * F + f] = from_float<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+  out[(size_t)n * F + f] = from_float<T>(clamped_swish_product(to_float(gu[(size_t)n * 2 * F + f]), to_float(gu[(size_t)n * 2 * F + F + f]), alpha, limit));
 }
 
 GIBBS_EXPORT int gibbs_glu_clamped(const void* gu, void* out, int dtype, int n, int F, float alpha, float limit, hipStream_t stream) {

@@ -63,6 +63,8 @@ int gibbs_skinny_residual(const void* X, const void* W, float* x, void* xb, int 
                           hipStream_t stream);
 int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw, long ldy, int rms,
                      float eps, int act, hipStream_t stream);
+int gibbs_skinny_glu_general(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw, long ldy, int rms,
+                             float eps, int act, float alpha, float limit, hipStream_t stream);
 int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N, int C, int I, long ldx, long ldw, int rms, float eps,
                       const float* taps, const float* bias, float* state, long slot_stride, const int* slot,
                       const int* ctx, int K, hipStream_t stream);

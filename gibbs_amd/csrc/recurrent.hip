@@ -8,6 +8,7 @@
 // recurrences walk a request's rows in order with a fixed order of additions per token, so a prompt
 // in one step, in portions or token by token gives the same bits.
 #include "common.h"
+#include "lane8.h"
 
 namespace {
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
@@ -134,13 +135,14 @@ struct RecurrenceArgs {
 // are on their way from memory into registers meanwhile.
 //   delta:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //   outer:  o = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T
-template <typename TIn, int RULE, int DPT, int PARTS>
+// CH: the decay is one per key channel (always so for the outer rule); else one per head.
+template <typename TIn, int RULE, int DPT, int PARTS, bool CH>
 __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
   constexpr int COLS = WAVE / PARTS, TOK = 8, DMAX = DPT * PARTS, LDP = DPT + 4, PER_LANE = TOK * DMAX / WAVE;
   constexpr int V_PER_LANE = (TOK * COLS + WAVE - 1) / WAVE;
   static_assert(DPT % 4 == 0 && TOK * DMAX % WAVE == 0, "a lane reads its channels four at a time");
   __shared__ __attribute__((aligned(16))) float sq[TOK][PARTS][LDP], sk[TOK][PARTS][LDP], sd[TOK][PARTS][LDP];
-  __shared__ float sv[TOK][COLS], sb[TOK], sg[TOK];
+  __shared__ float sv[TOK][COLS], sb[TOK], sg[TOK], so[TOK][COLS];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int col = lane / PARTS, part = lane % PARTS;
   const int j = blockIdx.z * COLS + col;
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
   const TIn* q = (const TIn*)a.q;
   const TIn* k = (const TIn*)a.k;
   const TIn* v = (const TIn*)a.v;
-  const bool channel_decay = RULE == RULE_OUTER || a.per_channel;
+  constexpr bool channel_decay = CH;
   // the next 8 tokens' operands, in registers until the current 8 are done with LDS
   float rq[PER_LANE], rk[PER_LANE], rd[PER_LANE], rv[V_PER_LANE], rb = 0.f, rg = 1.f;
   auto ask = [&](int t0) {
@@ -203,34 +205,49 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
       sg[lane] = rg;
     }
   };
-  auto fold = [&](float x) {
-#pragma unroll
-    for (int o = 1; o < PARTS; o <<= 1) x += __shfl_xor(x, o, WAVE);
-    return x;
+  // (the PARTS lanes of a column are neighbours within a row of 16 lanes: data-parallel moves, a few cycles each)
+  auto fold = [&](float x) { return group_sum<PARTS>(x); };
+  // The read-outs of 8 tokens leave together, right after the next tokens' operands have arrived and before the ones
+  // after them are asked for: whatever the wave then waits for in memory was asked a whole round of tokens ago.
+  auto flush = [&](int t0, int nt) {
+    for (int idx = lane; idx < TOK * COLS; idx += WAVE) {
+      const int t = idx / COLS, jj = blockIdx.z * COLS + idx % COLS;
+      if (t < nt && jj < V) a.out[(size_t)(first + t0 + t) * a.H * V + (size_t)h * V + jj] = so[t][idx % COLS];
+    }
   };
   if (rows > 0) ask(0);
   for (int t0 = 0; t0 < rows; t0 += TOK) {
     const int nt = min(TOK, rows - t0);
     __syncthreads();   // everyone is done with the tokens before
     put();
+    if (t0 > 0) flush(t0 - TOK, TOK);
     __syncthreads();
     if (t0 + TOK < rows) ask(t0 + TOK);
-    for (int t = 0; t < nt; ++t) {
-      const float vj = sv[t][col];
-      float kk[DPT], qq[DPT], dd[DPT];
+    // a token's operands are read from LDS while the token before it is worked on
+    float kk[DPT], qq[DPT], dd[DPT], vj, beta_t, g_head;
+    auto read = [&](int t, float (&k_)[DPT], float (&q_)[DPT], float (&d_)[DPT], float& v_, float& b_, float& g_) {
 #pragma unroll
       for (int c = 0; c < DPT / 4; ++c) {
         const float4 k4 = *(const float4*)&sk[t][part][c * 4], q4 = *(const float4*)&sq[t][part][c * 4];
-        kk[c * 4] = k4.x; kk[c * 4 + 1] = k4.y; kk[c * 4 + 2] = k4.z; kk[c * 4 + 3] = k4.w;
-        qq[c * 4] = q4.x; qq[c * 4 + 1] = q4.y; qq[c * 4 + 2] = q4.z; qq[c * 4 + 3] = q4.w;
+        k_[c * 4] = k4.x; k_[c * 4 + 1] = k4.y; k_[c * 4 + 2] = k4.z; k_[c * 4 + 3] = k4.w;
+        q_[c * 4] = q4.x; q_[c * 4 + 1] = q4.y; q_[c * 4 + 2] = q4.z; q_[c * 4 + 3] = q4.w;
         if (channel_decay) {
           const float4 d4 = *(const float4*)&sd[t][part][c * 4];
-          dd[c * 4] = d4.x; dd[c * 4 + 1] = d4.y; dd[c * 4 + 2] = d4.z; dd[c * 4 + 3] = d4.w;
+          d_[c * 4] = d4.x; d_[c * 4 + 1] = d4.y; d_[c * 4 + 2] = d4.z; d_[c * 4 + 3] = d4.w;
+        } else {
+          d_[c * 4] = d_[c * 4 + 1] = d_[c * 4 + 2] = d_[c * 4 + 3] = 1.f;
         }
       }
+      v_ = sv[t][col];
+      b_ = RULE == RULE_DELTA ? sb[t] : 0.f;
+      g_ = RULE == RULE_DELTA ? sg[t] : 1.f;
+    };
+    read(0, kk, qq, dd, vj, beta_t, g_head);
+    for (int t = 0; t < nt; ++t) {
+      float nk[DPT], nq[DPT], nd[DPT], nv, nb, ng;
+      read(min(t + 1, TOK - 1), nk, nq, nd, nv, nb, ng);
       float o0 = 0.f, o1 = 0.f;
       if (RULE == RULE_DELTA) {
-        const float g_head = sg[t];
         float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
@@ -239,7 +256,7 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
           dot0 = fmaf(S[ii], kk[ii], dot0);
           dot1 = fmaf(S[ii + 1], kk[ii + 1], dot1);
         }
-        const float u = sb[t] * (vj - fold(dot0 + dot1));
+        const float u = beta_t * (vj - fold(dot0 + dot1));
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
           S[ii] = fmaf(kk[ii], u, S[ii]);
@@ -258,8 +275,15 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
         }
       }
       const float o = fold(o0 + o1);
-      if (part == 0 && j < V) a.out[(size_t)(first + t0 + t) * a.H * V + (size_t)h * V + j] = o;
+      if (part == 0) so[t][col] = o;
+#pragma unroll
+      for (int ii = 0; ii < DPT; ++ii) { kk[ii] = nk[ii]; qq[ii] = nq[ii]; dd[ii] = nd[ii]; }
+      vj = nv; beta_t = nb; g_head = ng;
     }
+  }
+  if (rows > 0) {
+    __syncthreads();
+    flush((rows - 1) / TOK * TOK, rows - (rows - 1) / TOK * TOK);
   }
 #pragma unroll
   for (int ii = 0; ii < DPT; ++ii) {
@@ -269,12 +293,17 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
 }
 
 // Lanes per column by the key size: 8 channels a lane up to 128 channels, 16 beyond.
+template <typename TIn, int RULE, bool CH>
+void launch_recurrence_sized(const RecurrenceArgs& a, int n_req, hipStream_t stream) {
+  if (a.D <= 32) recurrence_kernel<TIn, RULE, 8, 4, CH><<<dim3(n_req, a.H, ceil_div(a.V, 16)), 64, 0, stream>>>(a);
+  else if (a.D <= 64) recurrence_kernel<TIn, RULE, 8, 8, CH><<<dim3(n_req, a.H, ceil_div(a.V, 8)), 64, 0, stream>>>(a);
+  else if (a.D <= 128) recurrence_kernel<TIn, RULE, 8, 16, CH><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
+  else recurrence_kernel<TIn, RULE, 16, 16, CH><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
+}
 template <typename TIn, int RULE>
 int launch_recurrence(const RecurrenceArgs& a, int n_req, hipStream_t stream) {
-  if (a.D <= 32) recurrence_kernel<TIn, RULE, 8, 4><<<dim3(n_req, a.H, ceil_div(a.V, 16)), 64, 0, stream>>>(a);
-  else if (a.D <= 64) recurrence_kernel<TIn, RULE, 8, 8><<<dim3(n_req, a.H, ceil_div(a.V, 8)), 64, 0, stream>>>(a);
-  else if (a.D <= 128) recurrence_kernel<TIn, RULE, 8, 16><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
-  else recurrence_kernel<TIn, RULE, 16, 16><<<dim3(n_req, a.H, ceil_div(a.V, 4)), 64, 0, stream>>>(a);
+  if (RULE == RULE_OUTER || a.per_channel) launch_recurrence_sized<TIn, RULE, true>(a, n_req, stream);
+  else launch_recurrence_sized<TIn, RULE, false>(a, n_req, stream);
   return 0;
 }
 

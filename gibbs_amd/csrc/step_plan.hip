@@ -46,7 +46,7 @@ long ceil_div_l(long a, long b) { return (a + b - 1) / b; }
 constexpr int FUSED_ROWS = 64;            // rows that the few-row products (and so the fused decode kernels) take
 constexpr int SKINNY_ROWS = 64;           // rows up to which a plain product takes the weight-streaming kernel
 constexpr int SKINNY_ROWS_F32_OUT = 48;   // the same for float32 output (the head: it streams faster than the tiled product)
-constexpr int ACT_CLAMPED = 4;            // the gated feed-forward's clamped activation (beside activation.h's codes 0 .. 3)
+constexpr int ACT_CLAMPED = 4;            // the gated feed-forward's clamped activation (activation.h: ACT_CLAMPED_SWISH)
 constexpr int MATRIX_SLICE_PAGES = 510;   // page ids of a key slice that the decode attention's matrix-core walk keeps in LDS
 
 // Ranges of k that the few-row product is cut into so that at least `want_blocks` workgroups run (a
@@ -578,14 +578,14 @@ struct GluBody : Body {
   Matrix gate_up, down;
   const void* gate_up_packed2 = nullptr;   // gate and up packed as two row groups, for the fused kernel
   int F = 0, act = 0;
-  // act ACT_CLAMPED: min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1); the stand-alone kernel only
+  // act ACT_CLAMPED: min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1)
   float alpha = 0.f, limit = 0.f;
-  bool fusable(bool) const override { return act != ACT_CLAMPED && gate_up.I % 8 == 0 && F % 8 == 0; }   // (rows one by one: any few rows)
+  bool fusable(bool) const override { return gate_up.I % 8 == 0 && F % 8 == 0; }   // (rows one by one: any few rows)
   void fused(Exec& e, float eps, float* x, void* mirror) const override {
     const int N = e.a.n_rows, H = gate_up.I;
     void* y = e.take((long)N * F * 2);
-    RUN(e, gibbs_skinny_glu(mirror, gate_up_packed2 ? gate_up_packed2 : gate_up.w, y, N, F, H, H, gate_up_packed2 ? 0 : H, F, 1, eps, act,
-                            e.a.stream));
+    RUN(e, gibbs_skinny_glu_general(mirror, gate_up_packed2 ? gate_up_packed2 : gate_up.w, y, N, F, H, H, gate_up_packed2 ? 0 : H, F, 1, eps,
+                                    act, alpha, limit, e.a.stream));
     e.skinny_residual(y, down, x, mirror);
     e.give(y);
   }

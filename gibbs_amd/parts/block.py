@@ -58,8 +58,12 @@ class ParallelNormsBlock(Block):
     Roles: `norm1`, then either `mixer`, or a pair of mixers `left` and `right` that read the same normed rows,
     each result normed over the width by `left_out` / `right_out` and the two averaged; `norm2` and `ffn` may
     be missing (a layer without a feed-forward).  The average's half is multiplied into the two out-norms'
-    gains when the weights are bound (exact: a power of two).  No gain is folded into matrices and no half of
-    this block takes the fused decode kernels: the step runs norm, body and add operations."""
+    gains when the weights are bound (exact: a power of two).
+
+    The feed-forward is laid down as a half of its own, x += ffn(norm2(x)), between the mixer's norm and the
+    mixer itself: the mixer's rows were normed before that half touched the stream, so both still read the
+    same x, and in bfloat16 the half takes the fused few-row kernels (norm2's gain folded into the gate and up
+    matrices) as a pre-norm block's does.  The mixers run norm, body and add operations."""
 
     def __init__(self, spec, hidden, layer_index):
         super().__init__(spec, hidden, layer_index)
@@ -75,9 +79,15 @@ class ParallelNormsBlock(Block):
         if self.pair:
             for norm in (self.left_out, self.right_out):
                 norm.gain = norm.gain * 0.5
+        if "ffn" in self.named and rt.act_dtype == torch.bfloat16:
+            if rt.fold_gains and hasattr(self.norm2, "fold_gain") and hasattr(self.ffn, "fold_input_gain"):
+                self.ffn.fold_input_gain(self.norm2.fold_gain())
+            self.ffn.pack_matrices()
 
     def emit(self, plan, caches) -> None:
         h = plan.normed(self.norm1.emit(plan))
+        if "ffn" in self.named:
+            plan.half(self.norm2.emit(plan), self.ffn.emit(plan))
         if self.pair:
             left = plan.apply(self.left.emit(plan, caches["left"]), h)
             right = plan.apply(self.right.emit(plan, caches["right"]), h)
@@ -85,9 +95,5 @@ class ParallelNormsBlock(Block):
         else:
             deltas = [plan.apply(self.mixer.emit(plan, caches["mixer"]), h)]
         plan.drop(h)
-        if "ffn" in self.named:
-            h2 = plan.normed(self.norm2.emit(plan))
-            deltas.append(plan.apply(self.ffn.emit(plan), h2))
-            plan.drop(h2)
         for d in deltas:
             plan.add(d)
