@@ -97,11 +97,11 @@ class AttentionMixer(Mixer):
             self.rot = self.position.rotation()
             self.slopes = self.position.score_slopes(self.heads)
             self.score_bias = self.position.score_table(self.heads)
+            self.pos_hook = self.rot is None and self.position.transforms_rows()
         # (the matrix-core kernels add the bias to unscaled scores, head by head)
         self.score_bias_over_scale = None
         if self.score_bias is not None and rt.act_dtype == torch.bfloat16 and self.scale > 0:
             self.score_bias_over_scale = (self.score_bias.t() / self.scale).contiguous()
-            self.pos_hook = self.rot is None and self.position.transforms_rows()
         if self.slopes is not None and (self.slopes.dtype != torch.float32 or tuple(self.slopes.shape) != (self.heads,)):
             raise ValueError(f"score slopes must be float32 [{self.heads}]")
 
