@@ -242,43 +242,48 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
       b_ = RULE == RULE_DELTA ? sb[t] : 0.f;
       g_ = RULE == RULE_DELTA ? sg[t] : 1.f;
     };
-    read(0, kk, qq, dd, vj, beta_t, g_head);
-    for (int t = 0; t < nt; ++t) {
-      float nk[DPT], nq[DPT], nd[DPT], nv, nb, ng;
-      read(min(t + 1, TOK - 1), nk, nq, nd, nv, nb, ng);
+    auto step = [&](int t, const float (&k_)[DPT], const float (&q_)[DPT], const float (&d_)[DPT], float v_, float b_, float g_) {
       float o0 = 0.f, o1 = 0.f;
       if (RULE == RULE_DELTA) {
         float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
-          S[ii] *= channel_decay ? dd[ii] : g_head;
-          S[ii + 1] *= channel_decay ? dd[ii + 1] : g_head;
-          dot0 = fmaf(S[ii], kk[ii], dot0);
-          dot1 = fmaf(S[ii + 1], kk[ii + 1], dot1);
+          S[ii] *= channel_decay ? d_[ii] : g_;
+          S[ii + 1] *= channel_decay ? d_[ii + 1] : g_;
+          dot0 = fmaf(S[ii], k_[ii], dot0);
+          dot1 = fmaf(S[ii + 1], k_[ii + 1], dot1);
         }
-        const float u = beta_t * (vj - fold(dot0 + dot1));
+        const float u = b_ * (v_ - fold(dot0 + dot1));
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
-          S[ii] = fmaf(kk[ii], u, S[ii]);
-          S[ii + 1] = fmaf(kk[ii + 1], u, S[ii + 1]);
-          o0 = fmaf(S[ii], qq[ii], o0);
-          o1 = fmaf(S[ii + 1], qq[ii + 1], o1);
+          S[ii] = fmaf(k_[ii], u, S[ii]);
+          S[ii + 1] = fmaf(k_[ii + 1], u, S[ii + 1]);
+          o0 = fmaf(S[ii], q_[ii], o0);
+          o1 = fmaf(S[ii + 1], q_[ii + 1], o1);
         }
       } else {
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
-          const float kv0 = kk[ii] * vj, kv1 = kk[ii + 1] * vj;
-          o0 = fmaf(qq[ii], fmaf(bonus[ii], kv0, S[ii]), o0);
-          o1 = fmaf(qq[ii + 1], fmaf(bonus[ii + 1], kv1, S[ii + 1]), o1);
-          S[ii] = fmaf(dd[ii], S[ii], kv0);
-          S[ii + 1] = fmaf(dd[ii + 1], S[ii + 1], kv1);
+          const float kv0 = k_[ii] * v_, kv1 = k_[ii + 1] * v_;
+          o0 = fmaf(q_[ii], fmaf(bonus[ii], kv0, S[ii]), o0);
+          o1 = fmaf(q_[ii + 1], fmaf(bonus[ii + 1], kv1, S[ii + 1]), o1);
+          S[ii] = fmaf(d_[ii], S[ii], kv0);
+          S[ii + 1] = fmaf(d_[ii + 1], S[ii + 1], kv1);
         }
       }
       const float o = fold(o0 + o1);
       if (part == 0) so[t][col] = o;
-#pragma unroll
-      for (int ii = 0; ii < DPT; ++ii) { kk[ii] = nk[ii]; qq[ii] = nq[ii]; dd[ii] = nd[ii]; }
-      vj = nv; beta_t = nb; g_head = ng;
+    };
+    // two sets of registers take turns: while one token is worked on, the next one's operands arrive in the other
+    float k2[DPT], q2[DPT], d2[DPT], v2, b2, g2;
+    read(0, kk, qq, dd, vj, beta_t, g_head);
+    for (int t = 0; t < nt; t += 2) {
+      read(min(t + 1, TOK - 1), k2, q2, d2, v2, b2, g2);
+      step(t, kk, qq, dd, vj, beta_t, g_head);
+      if (t + 1 < nt) {
+        read(min(t + 2, TOK - 1), kk, qq, dd, vj, beta_t, g_head);
+        step(t + 1, k2, q2, d2, v2, b2, g2);
+      }
     }
   }
   if (rows > 0) {
