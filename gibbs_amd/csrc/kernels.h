@@ -13,6 +13,8 @@ int gibbs_embed_general(const void* table, int dtype, const int* ids, float* x, 
                         float scale, const int* pos, const float* inv_freq, float* keep, hipStream_t stream);
 int gibbs_rmsnorm_rows(const void* in, int parts, long part_stride, const float* gain, float eps, void* out, int dtype, int n,
                        int hidden, hipStream_t stream);
+int gibbs_rmsnorm_rows_add(float* x, const void* in, int parts, long part_stride, const float* gain, float eps, int dtype, int n,
+                           int hidden, hipStream_t stream);
 int gibbs_glu_clamped(const void* gu, void* out, int dtype, int n, int F, float alpha, float limit, hipStream_t stream);
 int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
                                   const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
@@ -23,7 +25,7 @@ int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype,
                      float eps, int unit, float temp_coef, int temp_every, hipStream_t stream);
 int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
                            const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req, int C, int K,
-                           int update_state, hipStream_t stream);
+                           int update_state, int single_rows, hipStream_t stream);
 int gibbs_delta_prep(float* q, float* k, long ldqk, const void* beta_raw, const void* a_head, long ld_raw, int dtype,
                      const float* a_channel, const float* dt_bias, const float* a_log, float* beta, float* decay, int n_rows,
                      int G, int H, int D, float q_scale, float unit_eps, hipStream_t stream);
@@ -36,7 +38,7 @@ int gibbs_decayed_outer_rule(const void* r, const void* k, const void* v, int dt
 int gibbs_head_norm_gate(const float* o, const float* gain, int gain_len, const void* gate, long ld_gate, void* y, int dtype,
                          int n_rows, int H, int V, float eps, int act, hipStream_t stream);
 int gibbs_token_shift(const void* h, int dtype, const float* mu, int n_mix, float* state, long slot_stride, const int* row_req,
-                      const int* cu, const int* slot, void* out, int n_rows, int n_req, int W, int update_state,
+                      const int* cu, const int* slot, void* out, int n_rows, int n_req, int W, int update_state, int single_rows,
                       hipStream_t stream);
 int gibbs_tanh_rows(const float* in, void* out, int dtype, long count, hipStream_t stream);
 int gibbs_double_exp_decay(float* z, const float* bias, long count, int C, hipStream_t stream);

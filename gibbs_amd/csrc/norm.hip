@@ -230,6 +230,42 @@ __global__ void rmsnorm_rows_kernel(const void* __restrict__ in, int parts, size
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[at + i] = from_float<T>(gain ? value(i) * scale * gain[i] : value(i) * scale);
 }
 
+// The same added straight into the float32 stream: x += v * rsqrt(mean(v^2) + eps) * gain (no rounding of the normed rows).
+template <typename T>
+__global__ void rmsnorm_rows_add_kernel(float* __restrict__ x, const void* __restrict__ in, int parts, size_t part_stride,
+                                        const float* __restrict__ gain, float eps, int hidden) {
+  __shared__ float scratch[16];
+  const size_t at = (size_t)blockIdx.x * hidden;
+  auto value = [&](int i) -> float {
+    if (parts == 1) return to_float(((const T*)in)[at + i]);
+    float v = 0.f;
+    for (int s = 0; s < parts; ++s) v += ((const float*)in)[s * part_stride + at + i];
+    return v;
+  };
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = value(i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) x[at + i] += gain ? value(i) * scale * gain[i] : value(i) * scale;
+}
+
+GIBBS_EXPORT int gibbs_rmsnorm_rows_add(float* x, const void* in, int parts, long part_stride, const float* gain, float eps, int dtype,
+                                        int n, int hidden, hipStream_t stream) {
+  GIBBS_REQUIRE(x && in && n >= 0 && hidden > 0 && parts >= 1, "rmsnorm_rows_add: bad sizes n=%d hidden=%d parts=%d", n, hidden, parts);
+  if (n == 0) return 0;
+  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  if (dtype == GIBBS_F32)
+    rmsnorm_rows_add_kernel<float><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain, eps, hidden);
+  else if (dtype == GIBBS_BF16)
+    rmsnorm_rows_add_kernel<bf16><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain, eps, hidden);
+  else
+    return gibbs_fail("rmsnorm_rows_add: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("rmsnorm_rows_add");
+}
+
 GIBBS_EXPORT int gibbs_rmsnorm_rows(const void* in, int parts, long part_stride, const float* gain, float eps, void* out, int dtype,
                                     int n, int hidden, hipStream_t stream) {
   GIBBS_REQUIRE(in && out && n >= 0 && hidden > 0 && parts >= 1, "rmsnorm_rows: bad sizes n=%d hidden=%d parts=%d", n, hidden, parts);

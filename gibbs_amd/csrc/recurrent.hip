@@ -22,19 +22,22 @@ __device__ __forceinline__ float activate_gate(float z, int act) {   // 0: silu,
 // step's first row come from the request's state (its last K-1 inputs, oldest first; zeros at a sequence's start).
 template <typename T>
 __global__ void causal_conv_silu_kernel(const T* __restrict__ in, long ld, const float* __restrict__ taps,
-                                        const float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
+                                        float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
                                         const int* __restrict__ cu, const int* __restrict__ slot, float* __restrict__ out,
-                                        int C, int K) {
+                                        int C, int K, int shift_state) {
   const int n = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int r = row_req[n], first = cu[r], t = n - first;
-  const float* st = state + (size_t)slot[r] * slot_stride;
+  float* st = state + (size_t)slot[r] * slot_stride;
   float acc = 0.f;
   for (int j = 0; j < K; ++j) {
     const int tt = t - (K - 1) + j;
     const float xv = tt >= 0 ? to_float(in[(size_t)(first + tt) * ld + c]) : st[(size_t)(K - 1 + tt) * C + c];
     acc = fmaf(taps[(size_t)c * K + j], xv, acc);
+    // every request brings one row (shift_state): this thread is the only one that reads or writes the request's
+    // inputs of this channel, so it moves them on itself (entry j - 1 has been read already)
+    if (shift_state && j >= 1) st[(size_t)(j - 1) * C + c] = xv;
   }
   out[(size_t)n * C + c] = acc * sigmoid_f(acc);
 }
@@ -335,14 +338,16 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restr
 // before, or for a step's first row the request's state (zeros at a sequence's start).
 template <typename T>
 __global__ void token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int n_mix,
-                                   const float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
-                                   const int* __restrict__ cu, const int* __restrict__ slot, T* __restrict__ out, int N, int W) {
+                                   float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
+                                   const int* __restrict__ cu, const int* __restrict__ slot, T* __restrict__ out, int N, int W,
+                                   int keep_row) {
   const int n = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= W) return;
   const int r = row_req[n];
   const float cur = to_float(h[(size_t)n * W + c]);
   const float prev = n > cu[r] ? to_float(h[(size_t)(n - 1) * W + c]) : state[(size_t)slot[r] * slot_stride + c];
+  if (keep_row) state[(size_t)slot[r] * slot_stride + c] = cur;   // (every request brings one row: it is the next step's previous row)
   for (int s = 0; s < n_mix; ++s)
     out[((size_t)s * N + n) * W + c] = from_float<T>(fmaf(prev - cur, mu[(size_t)s * W + c], cur));
 }
@@ -376,14 +381,16 @@ __global__ void double_exp_decay_kernel(float* __restrict__ z, const float* __re
 
 GIBBS_EXPORT int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
                                         const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req,
-                                        int C, int K, int update_state, hipStream_t stream) {
+                                        int C, int K, int update_state, int single_rows, hipStream_t stream) {
+  // single_rows: every request brings exactly one row (a step of decoded tokens): the state moves on in the same kernel
+  const int shift = update_state && single_rows && K > 1 && n_rows == n_req;
   GIBBS_REQUIRE(in && taps && state && out && n_rows > 0 && n_req > 0 && C > 0 && K >= 1 && ld >= C && slot_stride >= (long)(K - 1) * C,
                 "causal_conv: bad operands rows=%d requests=%d C=%d K=%d", n_rows, n_req, C, K);
   const dim3 rows(n_rows, ceil_div(C, 256)), reqs(n_req, ceil_div(C, 256));
   BY_DTYPE(dtype, "causal_conv",
-           (causal_conv_silu_kernel<float><<<rows, 256, 0, stream>>>((const float*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K)),
-           (causal_conv_silu_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K)));
-  if (update_state && K > 1)
+           (causal_conv_silu_kernel<float><<<rows, 256, 0, stream>>>((const float*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K, shift)),
+           (causal_conv_silu_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K, shift)));
+  if (update_state && K > 1 && !shift)
     BY_DTYPE(dtype, "causal_conv",
              (causal_conv_state_kernel<float><<<reqs, 256, 0, stream>>>((const float*)in, ld, state, slot_stride, cu, slot, C, K)),
              (causal_conv_state_kernel<bf16><<<reqs, 256, 0, stream>>>((const bf16*)in, ld, state, slot_stride, cu, slot, C, K)));
@@ -446,14 +453,15 @@ GIBBS_EXPORT int gibbs_head_norm_gate(const float* o, const float* gain, int gai
 
 GIBBS_EXPORT int gibbs_token_shift(const void* h, int dtype, const float* mu, int n_mix, float* state, long slot_stride,
                                    const int* row_req, const int* cu, const int* slot, void* out, int n_rows, int n_req, int W,
-                                   int update_state, hipStream_t stream) {
+                                   int update_state, int single_rows, hipStream_t stream) {
+  const int keep = update_state && single_rows && n_rows == n_req;
   GIBBS_REQUIRE(h && mu && state && out && n_rows > 0 && n_req > 0 && W > 0 && n_mix > 0 && slot_stride >= W,
                 "token_shift: bad operands rows=%d requests=%d W=%d", n_rows, n_req, W);
   const dim3 rows(n_rows, ceil_div(W, 256)), reqs(n_req, ceil_div(W, 256));
   BY_DTYPE(dtype, "token_shift",
-           (token_shift_kernel<float><<<rows, 256, 0, stream>>>((const float*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (float*)out, n_rows, W)),
-           (token_shift_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (bf16*)out, n_rows, W)));
-  if (update_state)
+           (token_shift_kernel<float><<<rows, 256, 0, stream>>>((const float*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (float*)out, n_rows, W, keep)),
+           (token_shift_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)h, mu, n_mix, state, slot_stride, row_req, cu, slot, (bf16*)out, n_rows, W, keep)));
+  if (update_state && !keep)
     BY_DTYPE(dtype, "token_shift",
              (token_shift_state_kernel<float><<<reqs, 256, 0, stream>>>((const float*)h, state, slot_stride, cu, slot, W)),
              (token_shift_state_kernel<bf16><<<reqs, 256, 0, stream>>>((const bf16*)h, state, slot_stride, cu, slot, W)));

@@ -262,6 +262,8 @@ struct NormPart {
   virtual bool folded_rms(float* eps) const { return false; }
   // the norm of a part's result before it is added (the stream is not touched); gives the delta's buffer back
   virtual Pending run_on(Exec& e, Pending delta) const;
+  // x += norm(a part's result) in one pass, where the norm can (else: false, and nothing is done)
+  virtual bool add_normed(Exec& e, float* x, Pending delta) const { return false; }
 };
 
 struct Body {
@@ -289,7 +291,7 @@ struct Plan {
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
   std::vector<std::unique_ptr<NormPart>> norms;
   std::vector<std::unique_ptr<Body>> bodies;
-  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT };
+  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT, OP_ADD_NORMED };
   struct Op {
     int kind, norm, body, value;   // value: what a body reads, an add adds, a drop drops
     int result;                    // the value that a norm or a body makes
@@ -369,6 +371,12 @@ struct RmsNorm : NormPart {
   bool folded_rms(float* e) const override {
     *e = eps;
     return gain == nullptr;
+  }
+  bool add_normed(Exec& e, float* x, Pending delta) const override {
+    const int N = e.a.n_rows, H = e.p.hidden;
+    RUN(e, gibbs_rmsnorm_rows_add(x, delta.data, std::max(delta.parts, 1), (long)N * H, gain, eps, e.p.dtype, N, H, e.a.stream));
+    e.give(delta.data);
+    return true;
   }
   Pending run_on(Exec& e, Pending delta) const override {
     const int N = e.a.n_rows, H = e.p.hidden;
@@ -630,7 +638,7 @@ struct DeltaBody : Body {
     char* raw = (char*)e.linear(h, in, N, false, false, false, nullptr);
     float* qkv = (float*)e.take((long)N * C * 4);
     RUN(e, gibbs_causal_conv_silu(raw, in.O, e.p.dtype, taps, conv_state, slot_stride, a.row_req, a.cu, a.slot, qkv, N, a.n_req, C, K, 1,
-                                  a.stream));
+                                  a.max_q == 1, a.stream));
     float* a_channel = channel ? (float*)e.linear(raw + (long)off_a * e.esize, a2, N, true, false, false, nullptr, in.O) : nullptr;
     float* beta = (float*)e.take((long)N * H * 4);
     float* decay = (float*)e.take((long)N * H * (channel ? D : 1) * 4);
@@ -676,7 +684,8 @@ struct TimeMixBody : Body {
     const GibbsStepArgs& a = e.a;
     const int N = a.n_rows, W = e.p.hidden, C = H * D;
     char* mixes = (char*)e.take(5L * N * W * e.esize);
-    RUN(e, gibbs_token_shift(h, e.p.dtype, mu, 5, shift_state, slot_stride, a.row_req, a.cu, a.slot, mixes, N, a.n_req, W, 1, a.stream));
+    RUN(e, gibbs_token_shift(h, e.p.dtype, mu, 5, shift_state, slot_stride, a.row_req, a.cu, a.slot, mixes, N, a.n_req, W, 1, a.max_q == 1,
+                             a.stream));
     const long one = (long)N * W * e.esize;
     void* r = e.linear(mixes, wr, N, false, false, false, nullptr);
     void* k = e.linear(mixes + one, wk, N, false, false, false, nullptr);
@@ -776,6 +785,18 @@ void Exec::run() {
       case Plan::OP_NORM_DELTA:
         deltas[op.result] = p.norms[op.norm]->run_on(*this, deltas[op.value]);
         deltas[op.value] = Pending{};
+        break;
+      case Plan::OP_ADD_NORMED:
+        // (what is pending stays pending: additions into x commute, and the next norm still takes it on its way)
+        if (p.norms[op.norm]->add_normed(*this, x, deltas[op.value])) {
+          deltas[op.value] = Pending{};
+          give(mirror);
+          mirror = nullptr;
+        } else {
+          settle(x, pending);
+          pending = p.norms[op.norm]->run_on(*this, deltas[op.value]);
+          deltas[op.value] = Pending{};
+        }
         break;
       case Plan::OP_REINJECT:
         settle(x, pending);
@@ -1064,6 +1085,12 @@ GIBBS_EXPORT int gibbs_plan_op_norm_delta(void* plan, int norm, int value) {
   if (!p) return -1;
   if (!p->has_norm(norm) || !known_value(p, value)) { gibbs_fail("plan: norm %d of value %d: no such part or value", norm, value); return -1; }
   return append(p, Plan::OP_NORM_DELTA, norm, -1, value, true);
+}
+GIBBS_EXPORT int gibbs_plan_op_add_normed(void* plan, int norm, int value) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!p->has_norm(norm) || !known_value(p, value)) { gibbs_fail("plan: norm %d of value %d: no such part or value", norm, value); return -1; }
+  return append(p, Plan::OP_ADD_NORMED, norm, -1, value, false);
 }
 GIBBS_EXPORT int gibbs_plan_op_reinject(void* plan) {
   Plan* p = open_plan(plan);

@@ -116,6 +116,7 @@ int gibbs_plan_op_body(void* plan, int body, int value);      // -> value: body(
 int gibbs_plan_op_add(void* plan, int value);                 // x += delta (lazily: it stays pending for the next norm)
 int gibbs_plan_op_drop(void* plan, int value);                // the value is not read again
 int gibbs_plan_op_norm_delta(void* plan, int norm, int value);   // -> value: norm(a body's delta), the stream untouched
+int gibbs_plan_op_add_normed(void* plan, int norm, int value);   // x += norm(a body's delta), in one pass where the norm can
 int gibbs_plan_op_reinject(void* plan);                       // x += the embedding's output (what the step's first operation saw)
 int gibbs_plan_tail(void* plan, int norm);                    // the norm in front of the head
 int gibbs_plan_op_count(const void* plan);

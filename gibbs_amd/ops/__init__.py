@@ -540,7 +540,7 @@ def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, r
     _i32(row_req, n, "row_req"); _i32(cu, n_req + 1, "cu"); _i32(slot, n_req, "slot")
     out = torch.empty((n, c), dtype=torch.float32, device=x.device)
     call("gibbs_causal_conv_silu", ptr(x), c, dtype_code(x.dtype), ptr(taps), ptr(state), state.stride(0), ptr(row_req), ptr(cu),
-         ptr(slot), ptr(out), n, n_req, c, k, int(update_state), stream())
+         ptr(slot), ptr(out), n, n_req, c, k, int(update_state), int(n == n_req), stream())
     return out
 
 

@@ -91,9 +91,10 @@ class ParallelNormsBlock(Block):
         if self.pair:
             left = plan.apply(self.left.emit(plan, caches["left"]), h)
             right = plan.apply(self.right.emit(plan, caches["right"]), h)
-            deltas = [plan.normed_delta(self.left_out.emit(plan), left), plan.normed_delta(self.right_out.emit(plan), right)]
+            plan.drop(h)
+            plan.add_normed(self.left_out.emit(plan), left)      # (normed and added in float32, in one pass each)
+            plan.add_normed(self.right_out.emit(plan), right)
         else:
-            deltas = [plan.apply(self.mixer.emit(plan, caches["mixer"]), h)]
-        plan.drop(h)
-        for d in deltas:
-            plan.add(d)
+            delta = plan.apply(self.mixer.emit(plan, caches["mixer"]), h)
+            plan.drop(h)
+            plan.add(delta)

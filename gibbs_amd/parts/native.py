@@ -80,6 +80,7 @@ def declare(lib) -> None:
         "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
         "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
         "gibbs_plan_op_norm_delta": ([P, I, I], I),
+        "gibbs_plan_op_add_normed": ([P, I, I], I),
         "gibbs_plan_op_reinject": ([P], I),
         "gibbs_plan_op_half": ([P, I, I], I),
         "gibbs_plan_op_norm": ([P, I], I),
@@ -309,6 +310,10 @@ class NativePlan:
     def normed_delta(self, norm: int, value: int) -> int:
         """-> value: norm(a body's delta), before it is added; the stream is not touched."""
         return self._made(L.library().gibbs_plan_op_norm_delta(self.handle, norm, value))
+
+    def add_normed(self, norm: int, value: int) -> None:
+        """x += norm(a body's delta): normed and added in one pass (float32), the delta is used up."""
+        self._made(L.library().gibbs_plan_op_add_normed(self.handle, norm, value))
 
     def reinject(self) -> None:
         """x += the embedding's output (the rows as the step's first operation saw them)."""
