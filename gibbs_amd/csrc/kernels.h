@@ -22,7 +22,7 @@ int gibbs_attention_plain_general(const void* q, const void* kpages, const void*
                                   const float* slopes, const float* bias, int bias_len, hipStream_t stream);
 int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype, const int* pos, const int* row_req,
                      const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
-                     float eps, int unit, float temp_coef, int temp_every, hipStream_t stream);
+                     float eps, int unit, int norm_dim, float temp_coef, int temp_every, hipStream_t stream);
 int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
                            const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req, int C, int K,
                            int update_state, int single_rows, hipStream_t stream);

@@ -457,6 +457,7 @@ struct AttnBody : Body {
   // square without a gain, a temperature on q that grows with the position, a table of score biases over the distance
   int vd = 0;
   int unit_qk = 0, temp_every = 0;
+  int norm_dim = 0;                   // channels of a head that the unit norm's mean runs over (heads may be stored wider, zero-padded)
   float temp_coef = 0.f;
   const float* bias = nullptr;        // [bias_len, nh]
   const float* bias_t = nullptr;      // the same as [nh, bias_len] divided by the scale: what the matrix-core kernels add to raw scores
@@ -507,7 +508,7 @@ struct AttnBody : Body {
     const int width = e.width(group);
     if (extras()) {
       RUN(e, gibbs_qk_unit_kv(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, e.a.pos, e.a.row_req, table, width,
-                              page_size, num_pages, N, nh, kv, hd, vd, qk_eps, unit_qk, temp_coef, temp_every, e.a.stream));
+                              page_size, num_pages, N, nh, kv, hd, vd, qk_eps, unit_qk, norm_dim, temp_coef, temp_every, e.a.stream));
       return;
     }
     if (!hook) {
@@ -964,7 +965,7 @@ GIBBS_EXPORT int gibbs_plan_embedding(void* plan, float scale, const float* inv_
   return 0;
 }
 
-GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, float temp_coef, int temp_every,
+GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, int norm_dim, float temp_coef, int temp_every,
                                              const float* bias, const float* bias_t, int bias_len) {
   Plan* p = open_plan(plan);
   if (!p) return -1;
@@ -974,7 +975,7 @@ GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int u
     gibbs_fail("plan: an attention with these extras has no rotation, no q/k gains, no hook and no slopes, and owns its pages");
     return -1;
   }
-  t->vd = vd; t->unit_qk = unit_qk; t->temp_coef = temp_coef; t->temp_every = temp_every; t->bias = bias; t->bias_t = bias ? bias_t : nullptr; t->bias_len = bias ? bias_len : 0;
+  t->vd = vd; t->unit_qk = unit_qk; t->norm_dim = norm_dim > 0 ? norm_dim : t->hd; t->temp_coef = temp_coef; t->temp_every = temp_every; t->bias = bias; t->bias_t = bias ? bias_t : nullptr; t->bias_len = bias ? bias_len : 0;
   t->qkv.O = (t->nh + t->nkv) * t->hd + t->nkv * vd;
   t->out.I = t->nh * vd;
   return 0;

@@ -75,12 +75,13 @@ int gibbs_plan_body_host(void* plan, GibbsHostBody fn, void* user, int group);  
 // entry 2i = sin(pos * inv_freq[i]), entry 2i + 1 = cos of the same.
 int gibbs_plan_embedding(void* plan, float scale, const float* inv_freq);
 // An attention body without rotation and q/k gains may have: values of head size vd; q and k divided by their root
-// mean square per head (unit_qk, with the body's qk_eps); q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)
+// mean square per head (unit_qk, with the body's qk_eps; the mean over the first norm_dim channels of a head, which may
+// be stored wider with zeros behind them; 0: the head size); q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)
 // (temp_every 0: none); bias [bias_len, heads] added to the scores by distance (the last row for all longer ones),
 // and the same table as bias_t [heads, bias_len] divided by the scale (null: the matrix-core kernels are not used).
 // Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd].
-int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, float temp_coef, int temp_every, const float* bias,
-                                const float* bias_t, int bias_len);
+int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, int norm_dim, float temp_coef, int temp_every,
+                                const float* bias, const float* bias_t, int bias_len);
 // A gated feed-forward body computes min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1) instead.
 int gibbs_plan_glu_clamped(void* plan, int body, float alpha, float limit);
 

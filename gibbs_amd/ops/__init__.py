@@ -511,9 +511,10 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
 
 def qk_unit_kv(rows: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, *, kpages: Optional[torch.Tensor],
                vpages: Optional[torch.Tensor], table: Optional[torch.Tensor], pos: torch.Tensor, row_req: torch.Tensor,
-               eps: float, unit: bool = True, temp_coef: float = 0.0, temp_every: int = 0) -> None:
+               eps: float, unit: bool = True, temp_coef: float = 0.0, temp_every: int = 0, norm_dim: int = 0) -> None:
     """rows [N, nh*hd + nkv*hd + nkv*vd], in place: every head of q and k divided by its root mean square
-    (`unit`), q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1), k and v written to their pages."""
+    (`unit`; over the first `norm_dim` channels of a head when heads are stored wider, zero-padded), q times
+    1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1), k and v written to their pages."""
     require_cuda(rows, kpages, vpages, table, pos, row_req)
     n = rows.shape[0]
     assert rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] == (nh + nkv) * hd + nkv * vd
@@ -524,7 +525,7 @@ def qk_unit_kv(rows: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, *, kpage
         assert _check_pages(vpages, nkv, vd, rows.dtype) == (num_pages, page_size) and table.dtype == torch.int32 and table.is_contiguous()
         width = table.shape[1]
     call("gibbs_qk_unit_kv", ptr(rows), rows.shape[1], ptr(kpages), ptr(vpages), dtype_code(rows.dtype), ptr(pos), ptr(row_req),
-         ptr(table), width, page_size, num_pages, n, nh, nkv, hd, vd, float(eps), int(unit), float(temp_coef), int(temp_every), stream())
+         ptr(table), width, page_size, num_pages, n, nh, nkv, hd, vd, float(eps), int(unit), int(norm_dim), float(temp_coef), int(temp_every), stream())
 
 
 def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor, cu: torch.Tensor,

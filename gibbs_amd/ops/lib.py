@@ -58,7 +58,7 @@ _SIGNATURES = {
                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p,
                                       c_void_p, c_int, c_void_p],
     "gibbs_qk_unit_kv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int, c_void_p],
+                         c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_int, c_void_p],
     "gibbs_causal_conv_silu": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_delta_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p,

@@ -55,8 +55,25 @@ class AttentionMixer(Mixer):
     def cache_need(self) -> Optional[CacheNeed]:
         if self.source is not None:
             return None
-        return CacheNeed(self.kv_heads, self.head_dim, None if self.window is None else int(self.window),
-                         None if self.v_head_dim == self.head_dim else self.v_head_dim)
+        hd, vd = self.stored_dims()
+        return CacheNeed(self.kv_heads, hd, None if self.window is None else int(self.window), None if vd == hd else vd)
+
+    def stored_dims(self):
+        """(key, value) head sizes as projected and cached: the mixer's own, or, once it is bound for a bfloat16 run with
+        keys and values of different sizes (or sizes that are no multiple of 16), one common size with zeros behind each
+        head's channels, which the matrix-core attention kernels take."""
+        pad = getattr(self, "padded_dim", None)
+        return (pad, pad) if pad else (self.head_dim, self.v_head_dim)
+
+    def _pad_heads(self, w: torch.Tensor, heads: int, dim: int, pad: int, rows: bool) -> torch.Tensor:
+        """[heads * dim, in] -> [heads * pad, in] (rows) or [out, heads * dim] -> [out, heads * pad], zeros behind each head."""
+        if rows:
+            out = torch.zeros((heads, pad, w.shape[1]), dtype=w.dtype, device=w.device)
+            out[:, :dim] = w.view(heads, dim, w.shape[1])
+            return out.view(heads * pad, w.shape[1])
+        out = torch.zeros((w.shape[0], heads, pad), dtype=w.dtype, device=w.device)
+        out[:, :, :dim] = w.view(w.shape[0], heads, dim)
+        return out.view(w.shape[0], heads * pad)
 
     def attention_flops(self, keys: float) -> float:
         """Multiply-adds x 2 of scores and weighted values when the step's rows see `keys` keys in all."""
@@ -82,12 +99,28 @@ class AttentionMixer(Mixer):
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
         t = self.spec.tensors
+        wq, w_out = weights[t["q_proj"]], weights[t["out_proj"]]
+        # A bfloat16 run of an attention that takes the general preparation of its rows anyway (a unit norm, a score table)
+        # stores every head of q, k and v at one size that the matrix-core kernels take: a multiple of 16 that holds the
+        # larger of the two, zeros behind each head's channels (rows of zeros in the projections, columns of zeros in the
+        # out-projection: products with them are exactly zero).
+        self.padded_dim = None
+        pad = -(-max(self.head_dim, self.v_head_dim) // 16) * 16
+        if (rt.act_dtype == torch.bfloat16 and self.source is None and self.qk_norm == "unit" and pad <= 128
+                and (self.head_dim, self.v_head_dim) != (pad, pad)):
+            self.padded_dim = pad
+            wq = self._pad_heads(wq, self.heads, self.head_dim, pad, rows=True)
+            w_out = self._pad_heads(w_out, self.heads, self.v_head_dim, pad, rows=False)
         if self.source is None:
             # one product for q, k and v: rows [Wq; Wk; Wv]
-            self.w_qkv = torch.cat([weights[t["q_proj"]], weights[t["k_proj"]], weights[t["v_proj"]]], dim=0).contiguous()
+            wk, wv = weights[t["k_proj"]], weights[t["v_proj"]]
+            if self.padded_dim:
+                wk = self._pad_heads(wk, self.kv_heads, self.head_dim, pad, rows=True)
+                wv = self._pad_heads(wv, self.kv_heads, self.v_head_dim, pad, rows=True)
+            self.w_qkv = torch.cat([wq, wk, wv], dim=0).contiguous()
         else:
-            self.w_qkv = weights[t["q_proj"]]
-        self.w_out = weights[t["out_proj"]]
+            self.w_qkv = wq
+        self.w_out = w_out.contiguous()
         self.p_qkv = self.p_out = None
         self.q_gain = weights[t["q_norm"]] if self.qk_norm == "before" else None
         self.k_gain = weights[t["k_norm"]] if self.qk_norm == "before" and self.source is None else None
@@ -125,24 +158,26 @@ class AttentionMixer(Mixer):
         self.p_out = ops.PackedWeight(self.w_out)
 
     def extras(self) -> bool:
-        """Options that the plain kernels take and the matrix-core kernels do not."""
+        """Options that take the general preparation of the step's rows (no rotation, no gains)."""
         return (self.v_head_dim != self.head_dim or self.qk_norm == "unit" or self.q_temperature is not None
                 or self.score_bias is not None)
 
     def emit(self, plan, cache) -> int:
-        if cache.kpages is None or cache.vpages.shape[-1] != self.v_head_dim or cache.kpages.shape[-1] != self.head_dim:
+        hd, vd = self.stored_dims()
+        if cache.kpages is None or cache.vpages.shape[-1] != vd or cache.kpages.shape[-1] != hd:
             raise ValueError("the attention mixer's pages do not have its head sizes")
         hook = self.position.apply if self.pos_hook else None
-        body = self._emit_body(plan, cache, hook)
+        body = self._emit_body(plan, cache, hook, hd)
         if self.extras():
             temp = self.q_temperature or {"coef": 0.0, "every": 0}
-            plan.attention_extras(body, v_head_dim=self.v_head_dim, unit_qk=self.qk_norm == "unit", temp_coef=float(temp["coef"]),
-                                  temp_every=int(temp["every"]), bias=self.score_bias, bias_over_scale=self.score_bias_over_scale)
+            plan.attention_extras(body, v_head_dim=vd, unit_qk=self.qk_norm == "unit", temp_coef=float(temp["coef"]),
+                                  temp_every=int(temp["every"]), bias=self.score_bias, bias_over_scale=self.score_bias_over_scale,
+                                  norm_dim=self.head_dim)
         return body
 
-    def _emit_body(self, plan, cache, hook) -> int:
+    def _emit_body(self, plan, cache, hook, head_dim: int) -> int:
         return plan.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
-                              kv_heads=self.kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+                              kv_heads=self.kv_heads, head_dim=head_dim, scale=self.scale, window=self.window,
                               q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
                               kpages=cache.kpages, vpages=cache.vpages, group=cache.group, owns=self.source is None,
                               slopes=self.slopes, rows_hook=hook)

@@ -75,7 +75,7 @@ def declare(lib) -> None:
         "gibbs_plan_body_glu": ([P, P, P, P, P, I, I], I),
         "gibbs_plan_body_host": ([P, HOST_BODY, P, I], I),
         "gibbs_plan_embedding": ([P, F, P], I),
-        "gibbs_plan_attention_extras": ([P, I, I, I, F, I, P, P, I], I),
+        "gibbs_plan_attention_extras": ([P, I, I, I, I, F, I, P, P, I], I),
         "gibbs_plan_glu_clamped": ([P, I, F, F], I),
         "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
         "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
@@ -230,13 +230,14 @@ class NativePlan:
         return self._made(L.library().gibbs_plan_body_glu(self.handle, *ptrs, int(inter), int(activation)))
 
     def attention_extras(self, body: int, *, v_head_dim: int, unit_qk: bool, temp_coef: float, temp_every: int, bias,
-                         bias_over_scale=None) -> None:
+                         bias_over_scale=None, norm_dim: int = 0) -> None:
         """Options of an attention body without rotation: values of a head size of their own, q and k divided by
         their root mean square, a temperature on q, a table [distances, heads] of score biases (and the same as
         [heads, distances] divided by the score's scale, for the kernels that add it to unscaled scores)."""
         b, bt = self._held(bias, bias_over_scale)
-        self._made(L.library().gibbs_plan_attention_extras(self.handle, int(body), int(v_head_dim), int(unit_qk), float(temp_coef),
-                                                           int(temp_every), b, bt, 0 if bias is None else int(bias.shape[0])))
+        self._made(L.library().gibbs_plan_attention_extras(self.handle, int(body), int(v_head_dim), int(unit_qk), int(norm_dim),
+                                                           float(temp_coef), int(temp_every), b, bt,
+                                                           0 if bias is None else int(bias.shape[0])))
 
     def glu_clamped(self, body: int, *, alpha: float, limit: float) -> None:
         self._made(L.library().gibbs_plan_glu_clamped(self.handle, int(body), float(alpha), float(limit)))
