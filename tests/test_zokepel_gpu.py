@@ -267,6 +267,38 @@ def test_unit_norm_temperature_and_cache_write():
         assert np.array_equal(vp[page, :, p % ps].cpu().numpy().reshape(-1), before[i, (nh + nkv) * hd:])
 
 
+def test_heads_of_unequal_sizes_are_stored_padded_in_bfloat16_only(dirs):
+    """Keys of 24 and values of 40 (model P) run as heads of 48 in a bfloat16 engine (zeros behind each head's channels, in
+    the projections and in the pages: what the matrix-core attention kernels take) and at their own sizes in 32-bit; the
+    logits of both are held against the plain implementation by the tests above."""
+    for dtype, sizes in (("bfloat16", (48, 48)), ("float32", (24, 40))):
+        eng = make_engine(dirs["P"], dtype)
+        left = eng.model.blocks[1].left
+        assert left.stored_dims() == sizes and (left.head_dim, left.v_head_dim) == (24, 40)
+        group = eng.cache.group_needs.index(left.cache_need())
+        assert eng.device_cache.kpages[group].shape[-1] == sizes[0] and eng.device_cache.vpages[group].shape[-1] == sizes[1]
+        assert left.w_qkv.shape[0] == 6 * sizes[0] + 3 * sizes[0] + 3 * sizes[1] and left.w_out.shape[1] == 6 * sizes[1]
+        if dtype == "bfloat16":
+            q = left.w_qkv[:6 * 48].view(6, 48, -1)
+            assert float(q[:, 24:].abs().max()) == 0.0 and float(left.w_out.view(-1, 6, 48)[:, :, 40:].abs().max()) == 0.0
+
+
+def test_unit_norm_of_padded_heads_divides_by_the_true_size():
+    from gibbs_amd import ops
+    rng = np.random.default_rng(8)
+    nh, nkv, true, pad = 2, 1, 24, 32
+    rows = np.zeros((3, (nh + 2 * nkv) * pad), dtype=np.float32)
+    rows.reshape(3, nh + 2 * nkv, pad)[:, :, :true] = rng.normal(size=(3, nh + 2 * nkv, true))
+    dev = torch.tensor(rows, device="cuda")
+    pos = torch.tensor([0, 1, 2], dtype=torch.int32, device="cuda")
+    ops.qk_unit_kv(dev, nh, nkv, pad, pad, kpages=None, vpages=None, table=None, pos=pos, row_req=torch.zeros(3, dtype=torch.int32, device="cuda"),
+                   eps=1e-6, unit=True, norm_dim=true)
+    heads = rows.reshape(3, nh + 2 * nkv, pad)[:, :nh + nkv]
+    want = heads / np.sqrt((heads[:, :, :true] ** 2).mean(-1, keepdims=True) + 1e-6)
+    got = dev.cpu().numpy().reshape(3, nh + 2 * nkv, pad)[:, :nh + nkv]
+    assert np.allclose(got, want, rtol=2e-6, atol=1e-6) and np.abs(got[:, :, true:]).max() == 0.0
+
+
 @pytest.mark.parametrize("per_channel", [False, True])
 def test_delta_rule_keeps_an_old_write_through_portions_and_slots(per_channel):
     """A value written at the first token with a key of its own is read back 500 tokens later (no decay on that key's
