@@ -5,7 +5,7 @@
 
 enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_GELU = 2, ACT_RELU = 3, ACT_COUNT = 4 };
 // One more code, for gated products only: the clamped variant, which is no act(gate) * up:
-//   g = min(gate, limit), u = clamp(up, -limit, limit);  g * sigmoid(alpha * g) * (u + 1)
+//   the gate capped at `limit` from above, the up value clipped to +-limit; then gate * sigmoid(alpha * gate) * (1 + up)
 enum { ACT_CLAMPED_SWISH = 4 };
 __device__ __forceinline__ float clamped_swish_product(float gate, float up, float alpha, float limit) {
   const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);

@@ -1,8 +1,8 @@
 // Token embedding: x[n, :] = float(table[ids[n], :]) * scale (+ a sinusoidal position vector).  The
 // residual stream is float32 whatever the table's type is.
 //
-// The position vector, when `inv_freq` [hidden / 2] is given: entry 2i = sin(p * inv_freq[i]), entry
-// 2i + 1 = cos of the same angle, the angle being the float32 product of the float32 position and the
+// The position vector, when `inv_freq` [hidden / 2] is given: with a_i = p * inv_freq[i], even entries
+// 2i take sin(a_i) and odd entries 2i + 1 take cos(a_i), a_i being the float32 product of the float32 position and the
 // float32 frequency.  `keep` (optional) receives a second copy of the rows, for a model that adds the
 // embedding's output into the stream again later.
 #include "common.h"

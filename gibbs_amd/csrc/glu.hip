@@ -33,7 +33,7 @@ __global__ void glu_bf16x8_kernel(const bf16* __restrict__ gu, bf16* __restrict_
   *(uint4*)(out + (size_t)n * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-// The clamped variant:  g = min(gate, limit), u = clamp(up, -limit, limit);  out = g * sigmoid(alpha * g) * (u + 1).
+// The clamped variant (activation.h: the gate capped from above, the up value clipped, gate * sigmoid(alpha * gate) * (1 + up)).
 template <typename T>
 __global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float alpha, float limit) {
   const int n = blockIdx.x;

@@ -1,7 +1,7 @@
 // What an attention without rotation does to a step's projected rows before the scores: every head of q and
 // k is divided by its root mean square (an RMS norm without a gain: x / sqrt(mean(x^2) + eps)), q is
 // multiplied by a temperature that grows with the logarithm of the position,
-//     1 + coef * ln(floor((p + 1) / every) + 1),
+//     1 + coef * log(1 + (p + 1) div every)        (div: integer division),
 // and k and v go to their pages.  Values may have a head size of their own.  Rows are [q: nh*hd | k: nkv*hd |
 // v: nkv*vd]; q and k are changed in place (the attention kernel reads q from the row).  Sums, roots and
 // the temperature are float32.  Heads may be stored wider than they are (zeros behind their norm_dim channels, so

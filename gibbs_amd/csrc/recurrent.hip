@@ -77,7 +77,7 @@ struct DeltaPrepArgs {
 };
 
 // Block y < G: q and k of kv head y become unit vectors x / sqrt(sum x^2 + eps) (q times q_scale).  Block
-// y >= G: head y - G's beta = sigmoid(.) and decay g = exp(-exp(A_log) * softplus(a + dt_bias)).
+// y >= G: head y - G's beta = sigmoid(.) and decay = exp(-rate * softplus(a + dt_bias)) with rate = exp(A_log).
 template <typename T>
 __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaPrepArgs a) {
   const int n = blockIdx.x, lane = threadIdx.x;
@@ -136,8 +136,9 @@ struct RecurrenceArgs {
 // token waits for the one before, and what fills the chip is the number of independent chains.  Sums over the
 // key channels are folded over the PARTS lanes.  The operands of 8 tokens at a time go through LDS; the next 8
 // are on their way from memory into registers meanwhile.
-//   delta:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
-//   outer:  o = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T
+// With M the state [D, V], ' for transposed and .* for element by element along the key channels:
+//   delta:  M = decay * M;  w = beta * (v - M' k);  M = M + k w';  read = M' q
+//   outer:  read = (M + (bonus .* k) v')' r;  M = decay .* M (row by row) + k v'
 // CH: the decay is one per key channel (always so for the outer rule); else one per head.
 template <typename TIn, int RULE, int DPT, int PARTS, bool CH>
 __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
@@ -360,7 +361,7 @@ __global__ void token_shift_state_kernel(const T* __restrict__ h, float* __restr
   state[(size_t)slot[r] * slot_stride + c] = to_float(h[(size_t)(cu[r + 1] - 1) * W + c]);
 }
 
-// out = tanh(in) (float32 in, the activation type out); and w = exp(-exp(z + w0)) in place.
+// out = tanh(in) (float32 in, the activation type out); and decay = exp(-exp(z + bias)) in place.
 template <typename T>
 __global__ void tanh_kernel(const float* __restrict__ in, T* __restrict__ out, long count) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -428,7 +429,7 @@ GIBBS_EXPORT int gibbs_delta_rule(const float* q, const float* k, long ldqk, con
   GIBBS_LAUNCH_STATUS("delta_rule");
 }
 
-// o_t = (S + diag(bonus) k v^T)^T r; S <- diag(w) S + k v^T; r, k, v [N, H*D] in the activation type, w float32.
+// The decayed outer-product rule (see recurrence_kernel) over a ragged batch; r, k, v [N, H*D] in the activation type, w float32.
 GIBBS_EXPORT int gibbs_decayed_outer_rule(const void* r, const void* k, const void* v, int dtype, const float* w, const float* bonus,
                                           float* state, long slot_stride, const int* cu, const int* slot, float* out, int n_req,
                                           int H, int D, hipStream_t stream) {

@@ -668,7 +668,7 @@ struct DeltaBody : Body {
 
 // ---- time mixing with a decayed outer-product state
 // Each of r, k, v, g, w reads its own mix of the row and the row before it, h + (h' - h) mu_s; the decay is
-// w = exp(-exp(W2 tanh(W1 mix_w) + w0)); the rule runs over the requests' states S [heads, D, D]; each head's
+// decay = exp(-exp(z)), z = w0 + W2 tanh(W1 mix_w); the rule runs over the requests' states S [heads, D, D]; each head's
 // read-out is divided by its root mean square, multiplied by a gain and silu(g), and projected back.
 struct TimeMixBody : Body {
   Matrix wr, wk, wv, wg, w1, w2, out;

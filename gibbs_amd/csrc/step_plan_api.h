@@ -72,11 +72,11 @@ int gibbs_plan_body_glu(void* plan, const void* w_gate_up, const void* p_gate_up
 int gibbs_plan_body_host(void* plan, GibbsHostBody fn, void* user, int group);   // group: the cache group it reads, or -1
 
 // The embedding: rows of the table times `scale`, plus (inv_freq [hidden / 2] not null) a sinusoidal position vector,
-// entry 2i = sin(pos * inv_freq[i]), entry 2i + 1 = cos of the same.
+// sin(pos * inv_freq[i]) at the even entries 2i and the cosines of the same angles at the odd entries 2i + 1.
 int gibbs_plan_embedding(void* plan, float scale, const float* inv_freq);
 // An attention body without rotation and q/k gains may have: values of head size vd; q and k divided by their root
 // mean square per head (unit_qk, with the body's qk_eps; the mean over the first norm_dim channels of a head, which may
-// be stored wider with zeros behind them; 0: the head size); q times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)
+// be stored wider with zeros behind them; 0: the head size); q times 1 + temp_coef * log(1 + (pos + 1) div temp_every)
 // (temp_every 0: none); bias [bias_len, heads] added to the scores by distance (the last row for all longer ones),
 // and the same table as bias_t [heads, bias_len] divided by the scale (null: the matrix-core kernels are not used).
 // Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd].

@@ -514,7 +514,7 @@ def qk_unit_kv(rows: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, *, kpage
                eps: float, unit: bool = True, temp_coef: float = 0.0, temp_every: int = 0, norm_dim: int = 0) -> None:
     """rows [N, nh*hd + nkv*hd + nkv*vd], in place: every head of q and k divided by its root mean square
     (`unit`; over the first `norm_dim` channels of a head when heads are stored wider, zero-padded), q times
-    1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1), k and v written to their pages."""
+    1 + temp_coef * log(1 + (pos + 1) div temp_every), k and v written to their pages."""
     require_cuda(rows, kpages, vpages, table, pos, row_req)
     n = rows.shape[0]
     assert rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] == (nh + nkv) * hd + nkv * vd
@@ -566,7 +566,7 @@ def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Te
 
 def decayed_outer_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor, bonus: torch.Tensor, state: torch.Tensor,
                        cu: torch.Tensor, slot: torch.Tensor, heads: int) -> torch.Tensor:
-    """o_t = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T, per head over ragged rows: r, k, v [N, heads*D] in
+    """The decayed outer-product rule, read = (M + (bonus .* k) v')' r and then M = w .* M (row by row) + k v', per head over ragged rows: r, k, v [N, heads*D] in
     one type, w float32 [N, heads*D], bonus float32 [heads, D]; state [slots, heads, D, D] float32.  -> float32 [N, heads*D]."""
     require_cuda(r, k, v, w, bonus, state, cu, slot)
     n, c = r.shape

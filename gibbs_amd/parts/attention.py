@@ -38,7 +38,7 @@ class AttentionMixer(Mixer):
         self.qk_norm_eps = float(p.get("qk_norm_eps", 0.0))
         self.source = p.get("kv_source")
         # values of a head size of their own; q and k divided by their root mean square without a gain
-        # (`qk_norm: "unit"`); q times 1 + coef * ln(floor((position + 1) / every) + 1) (`q_temperature`)
+        # (`qk_norm: "unit"`); q times 1 + coef * log(1 + (position + 1) div every) (`q_temperature`)
         self.v_head_dim = int(p.get("v_head_dim") or self.head_dim)
         self.q_temperature = p.get("q_temperature")
         if self.heads % self.kv_heads:

@@ -3,15 +3,15 @@
 q = W_q h, k = W_k h (kv_heads x dim), v = W_v h (heads x vdim); each passes a short causal convolution
 per channel (taps [channels, K], the last one the current token's, zeros before a sequence's start) and
 silu; every head of q and k becomes a unit vector x / sqrt(sum x^2 + unit_eps), q times q_scale.  Per head
-(head h reads q/k head h // (heads / kv_heads)), with the state S [dim, vdim] starting at zero:
+(head h reads q/k head h // (heads / kv_heads)), with the state M [dim, vdim] starting at zero and ' for transposed:
 
-    S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+    M = decay * M;  w = beta * (v - M' k);  M = M + k w';  read = M' q
 
-beta = sigmoid(W_b h); the decay g = exp(-exp(A_log) softplus(a + dt_bias)) is one per head (`decay:
-"head"`, a = W_a h) or one per head and key channel, acting on the rows of S (`decay: "channel"`, a =
-W_a2 (W_a1 h), a low-rank pair).  Each head's o is divided by its root mean square, multiplied by a gain
+beta = sigmoid(W_b h); the decay, exp(-rate softplus(a + dt_bias)) with rate = exp(A_log), is one per head (`decay:
+"head"`, a = W_a h) or one per head and key channel, acting on the rows of M (`decay: "channel"`, a =
+W_a2 (W_a1 h), a low-rank pair).  Each head's read-out is divided by its root mean square, multiplied by a gain
 [vdim] shared by the heads and by a gate, silu(W_g h) (`gate: "silu"`) or sigmoid(W_g2 (W_g1 h)) (`gate:
-"sigmoid"`), and projected by W_o.  The state S and the convolutions' last K - 1 inputs live in the
+"sigmoid"`), and projected by W_o.  The state M and the convolutions' last K - 1 inputs live in the
 request's slot as float32; decays, beta, the unit vectors and the rule itself are float32 in both
 precisions of a run.  The kernels are csrc/recurrent.hip's; the step lays them out in csrc/step_plan.hip.
 """

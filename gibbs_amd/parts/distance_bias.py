@@ -3,8 +3,8 @@
 The table has B rows (one per bucket) and a column per head; a query at position i adds table[bucket(i - j), h]
 to its score with the key at position j.  With D the reach of the buckets:
 
-    bucket(n) = n                                                                    for n < B // 2
-              = min(B - 1, B // 2 + floor(ln(n / (B // 2)) / ln(D / (B // 2)) * (B - B // 2)))   otherwise
+    bucket(n) = n                                                     for n < h,      h = B // 2
+              = min(B - 1, h + floor((B - h) * log(n / h) / log(D / h)))   from h on
 
 so near distances have a bucket each, farther ones share buckets whose width grows with the distance, and
 every distance from D on has the last one.  The attention kernels get the bias as a table over the distance

@@ -2,8 +2,8 @@
 SwiGLU (arch/lib/transformer.json5:117-130, src/graph/cpu.rs:378-390).
 Gate and up are one product against [W_gate; W_up].
 
-`activation: "clamped_swish"` (with `limit` and `alpha`) is the clamped variant: g = min(gate, limit), u =
-clamp(up, -limit, limit), down(g * sigmoid(alpha * g) * (u + 1))."""
+`activation: "clamped_swish"` (with `limit` and `alpha`) is the clamped variant: the gate capped at `limit`
+from above, the up projection clipped to +-limit, down(gate * sigmoid(alpha * gate) * (1 + up))."""
 from __future__ import annotations
 
 from typing import List

@@ -95,7 +95,7 @@ class DecoderModel(Part):
         if pos is not None and pos.kind != "none":
             if pos.kind != "sinusoidal":
                 raise ValueError(f"position vector of kind {pos.kind!r} on the embedding is not implemented ('sinusoidal')")
-            # entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i) with f_i = base^(-2i / width), rounded to float32 once
+            # frequencies f_i = base^(-2i / width), rounded to float32 once; the kernel puts sin(p f_i) at 2i and cos(p f_i) at 2i + 1
             width = self.spec.hidden
             i = torch.arange(width // 2, dtype=torch.float64)
             self.embedding_inv_freq = (float(pos.params.get("base", 10000.0)) ** (-2.0 * i / width)).to(torch.float32).to(rt.device)

@@ -2,13 +2,13 @@
 
 With h' the previous token's row (zeros for a sequence's first token), each of r, k, v, g, w reads its own
 mix h + (h' - h) mu_s.  r, k, v = W_r, W_k, W_v of their mixes (heads x dim); gate = silu(W_g mix_g); the
-decay w = exp(-exp(W_2 tanh(W_1 mix_w) + w0)) per head and key channel.  Per head, with the state S [dim,
-dim] starting at zero and a bonus u [dim] for the current token only:
+decay is exp(-exp(z)) with z = w0 + W_2 tanh(W_1 mix_w), per head and key channel.  Per head, with the state M [dim,
+dim] starting at zero, ' for transposed, .* along the key channels, and a bonus [dim] for the current token only:
 
-    o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t;     S_t = diag(w_t) S_(t-1) + k_t v_t^T
+    read = (M + (bonus .* k) v')' r;  M = decay .* M (row by row) + k v'
 
-Each head's o is divided by its root mean square; the heads side by side are multiplied by a gain and the
-gate, and projected by W_o.  The state S and the previous token's row live in the request's slot as
+Each head's read-out is divided by its root mean square; the heads side by side are multiplied by a gain and the
+gate, and projected by W_o.  The state M and the previous token's row live in the request's slot as
 float32; the decay and the rule are float32 in both precisions of a run.  The kernels are
 csrc/recurrent.hip's; the step lays them out in csrc/step_plan.hip.
 """

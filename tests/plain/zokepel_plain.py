@@ -47,8 +47,8 @@ def unit_vector(x):
 
 # --------------------------------------------------------------------------- embedding
 def sinusoid(positions, width: int) -> np.ndarray:
-    """[T, width]: entry 2i = sin(p * 10000^(-2i/width)), entry 2i+1 = cos of the same angle; the
-    angle is a float32 product of the float32 position and the float32 frequency."""
+    """[T, width]: with f_i = 10000^(-2i/width) and a = p * f_i, out[p, 2i] = sin(a) and out[p, 2i+1] = cos(a); the
+    angle a is a float32 product of the float32 position and the float32 frequency."""
     i = np.arange(width // 2, dtype=F64)
     freq = (10000.0 ** (-2.0 * i / width)).astype(np.float32)
     angle = (np.asarray(positions, dtype=np.float32)[:, None] * freq[None, :]).astype(np.float32).astype(F64)
@@ -87,8 +87,8 @@ def causal_conv(x, taps) -> np.ndarray:
 # --------------------------------------------------------------------------- gated delta rule
 def delta_rule(q, k, v, beta, g) -> np.ndarray:
     """One head.  q, k [T, D]; v [T, V]; beta [T]; g [T] (one decay for the head) or [T, D] (one per key
-    channel, acting on the rows of S).  S [D, V] starts at zero; per token: S <- g S; u = beta (v - S^T k);
-    S <- S + k u^T; o = S^T q."""
+    channel, acting on the rows of the state).  The state M [D, V] starts at zero; per token, in this order:
+    M = g * M;  w = beta * (v - M' k);  M = M + k w';  out = M' q  (the read-out sees the token's own write)."""
     T, D = q.shape
     V = v.shape[1]
     S = np.zeros((D, V), dtype=F64)

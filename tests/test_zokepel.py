@@ -137,7 +137,7 @@ def test_plain_conv_and_feed_forward():
     assert np.allclose(y[:, 1], x[:, 1]) and y[0, 0] == 0 and y[1, 0] == 200 + 0 and y[2, 0] == 400 + 20 + 0
     h = np.array([[1.0, -2.0]])
     eye = np.eye(2)
-    big = Z.clamped_glu(h * 10, eye, eye, eye, 1.5)            # gate 10 -> 1.5; up -20 -> -1.5: y = g sigmoid(1.702 g) (u + 1)
+    big = Z.clamped_glu(h * 10, eye, eye, eye, 1.5)            # gate 10 -> 1.5; up -20 -> -1.5, then gate * sigmoid(1.702 gate) * (1 + up)
     assert np.allclose(big[0, 0], 1.5 * Z.sigmoid(1.702 * 1.5) * 2.5)
     assert np.allclose(big[0, 1], -20 * Z.sigmoid(1.702 * -20) * (-0.5))    # the gate is clamped from above only
     assert math.isclose(Z.sinusoid([3], 4)[0, 1], math.cos(3.0), rel_tol=1e-6) and Z.sinusoid([0], 6)[0].tolist() == [0, 1, 0, 1, 0, 1]
