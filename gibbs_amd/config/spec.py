@@ -15,10 +15,11 @@ from typing import Any, Mapping, Optional, Sequence, Tuple, Union
 
 @dataclass(frozen=True)
 class NormSpec:
-    """A normalisation over the last axis. `kind` selects the part (`"rms"`)."""
+    """A normalisation over the last axis. `kind` selects the part (`"rms"`; `"layer"`: mean taken off, gain and bias)."""
     kind: str
     eps: float
     weight: str                     # tensor name of the gain
+    bias: Optional[str] = None      # tensor name of the bias (kinds that have one)
 
 
 @dataclass(frozen=True)
@@ -51,7 +52,30 @@ class FeedForwardSpec:
     tensors: Mapping[str, str]
 
 
-PartSpec = Union[NormSpec, MixerSpec, FeedForwardSpec]
+@dataclass(frozen=True)
+class ConnectionSpec:
+    """How a sublayer reads and writes a model's residual streams (`"hyper"`: it reads a weighted sum of the
+    streams and writes every stream as a mix of the old ones plus a multiple of its result).  `tensors` maps the
+    part's roles (`"in"`, `"mix"`, `"out"`) to checkpoint names."""
+    kind: str
+    streams: int
+    tensors: Mapping[str, str]
+
+
+@dataclass(frozen=True)
+class EmbeddingTablesSpec:
+    """Rows of further tables that are added to the token table's row: `pair` [buckets + 1, width], row
+    (previous token * mul_prev + token * mul_cur) mod buckets, and row `buckets` for a sequence's first token;
+    `position` [positions, width], row = the token's position.  Either may be None."""
+    pair: Optional[str] = None
+    buckets: int = 0
+    mul_prev: int = 0
+    mul_cur: int = 0
+    position: Optional[str] = None
+    positions: int = 0
+
+
+PartSpec = Union[NormSpec, MixerSpec, FeedForwardSpec, ConnectionSpec]
 
 
 class LayerSpec:
@@ -119,3 +143,10 @@ class ModelSpec:
     embedding_scale: float = 1.0
     embedding_position: Optional[PositionSpec] = None
     reinject_before: Tuple[int, ...] = ()
+    # Tables whose rows are added to the token table's (hashed token pairs, learned positions), and the number of
+    # residual streams (every stream starts as the embedding's output; the model's output is their sum).
+    embedding_tables: Optional[EmbeddingTablesSpec] = None
+    streams: int = 1
+    # (name, shape) of checkpoint tensors that belong to the model and that no part reads (a layer without a
+    # feed-forward whose checkpoint holds that sublayer's norm all the same)
+    unread_tensors: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()

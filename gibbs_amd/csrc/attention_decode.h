@@ -99,7 +99,8 @@ __device__ __forceinline__ float load_through(const float* p) {
 // out = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s, eight slices' loads in flight at a time.
 // C: elements of a head per lane.
 template <int C>
-__device__ __forceinline__ void merge_slices_through(const float* ps, int n_splits, int hd, bf16* o, int lane) {
+__device__ __forceinline__ void merge_slices_through(const float* ps, int n_splits, int hd, bf16* o, int lane,
+                                                     const float* sink_of_head) {
   const int stride = hd + 2;
   float M = -INFINITY, L = 0.f, v[C];
 #pragma unroll
@@ -134,6 +135,7 @@ __device__ __forceinline__ void merge_slices_through(const float* ps, int n_spli
     }
     M = Mn;
   }
+  if (sink_of_head) L += __expf(*sink_of_head - M);   // (a sink counts once, whatever the number of slices)
   const float inv = 1.0f / L;
 #pragma unroll
   for (int c = 0; c < C; ++c) {
@@ -171,6 +173,8 @@ struct DecodeArgs {
   // positions back (the last entry for all farther ones), divided by `scale` already
   const float* bias;
   int bias_len;
+  // a sink per head, or null: [nh]; the softmax's denominator also holds exp(sink[h]) (natural units, not scaled)
+  const float* sink;
 };
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -579,6 +583,7 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
       const int head = kvh * G + g0 + g;
       if (a.n_splits == 1) {
         if (active) {
+          if (a.sink) ll += __expf(a.sink[head] - mm);
           const float inv = 1.0f / ll;
           bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
 #pragma unroll
@@ -622,7 +627,7 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   for (int g = wave; g < gcount; g += NW) {
     const int head = kvh * G + g0 + g;
     merge_slices_through<C>(partial + ((size_t)row * a.nh + head) * a.n_splits * (hd + 2), a.n_splits, hd,
-                            out + (size_t)row * a.ldo + (size_t)head * hd, lane);
+                            out + (size_t)row * a.ldo + (size_t)head * hd, lane, a.sink ? a.sink + head : nullptr);
   }
 }
 
@@ -693,7 +698,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
   if (a.n_splits > 1 && !a.merge_here) {
     dim3 mgrid(n_rows, ceil_div(a.nh, 4));
-    launch_attention_merge(mgrid, stream, partial, out, a.nh, a.hd, a.n_splits, a.ldo);
+    launch_attention_merge(mgrid, stream, partial, out, a.nh, a.hd, a.n_splits, a.ldo, a.sink);
   }
   GIBBS_LAUNCH_STATUS("attention_decode");
 }

@@ -41,6 +41,13 @@ int gibbs_attention_decode_bias(const void* q, const void* kpages, const void* v
                                 int nh, int nkv, int hd, long ldq, long ldo, float scale, int window, int n_splits, int waves,
                                 int kind, int max_keys, const float* bias, int bias_len, hipStream_t stream);
 
+// The same with a sink per head: float32 [nh] (null: none), a term exp(sink[h]) in the softmax's denominator that has no
+// key and no value and is not scaled; it counts once, whatever the number of key slices.
+int gibbs_attention_decode_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial, const int* pos,
+                                const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
+                                int nh, int nkv, int hd, long ldq, long ldo, float scale, int window, int n_splits, int waves,
+                                int kind, int max_keys, const float* bias, int bias_len, const float* sink, hipStream_t stream);
+
 // Floats of the per-GPU array behind gibbs_attention_decode_static (2 Mi floats = 8 MiB).
 long gibbs_attention_decode_static_capacity(void);
 

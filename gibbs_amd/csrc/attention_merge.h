@@ -1,6 +1,7 @@
 // The kernel that merges the key slices of an attention call: every slice of a (row, head) left
 // (max of the scaled scores, sum of exp(score - max), values weighted by exp(score - max)) as hd + 2
-// floats at partial[((row * heads + head) * slices + slice) * (hd + 2)].
+// floats at partial[((row * heads + head) * slices + slice) * (hd + 2)].  A sink per head (sink [heads], or null) adds
+// exp(sink[head]) to the merged sum, once.
 #pragma once
 #include "common.h"
 
@@ -13,7 +14,7 @@ namespace {
 // C: elements of a head per lane (head sizes up to 64 C); MERGE_AT_ONCE: slices merged with all loads at once.
 template <int C, int MERGE_AT_ONCE>
 __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int nh, int hd,
-                                       int n_splits, long ldo) {
+                                       int n_splits, long ldo, const float* __restrict__ sink) {
   const int row = blockIdx.x, head = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
   if (head >= nh) return;
@@ -47,6 +48,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
 #pragma unroll
       for (int c = 0; c < C; ++c) v[c] = fmaf(w, av[j][c], v[c]);
     }
+    if (sink) L += __expf(sink[head] - M);   // (a sink counts once, whatever the number of slices)
     const float inv = 1.0f / L;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
@@ -70,6 +72,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
     }
     L += wave_sum(term);
   }
+  if (sink) L += __expf(sink[head] - M);
   const float inv = 1.0f / L;
   for (int e = lane; e < hd; e += WAVE) {
     float v = 0.f;
@@ -92,12 +95,12 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
 
 // grid: (rows, ceil(heads / 4)), 4 waves a workgroup
 inline void launch_attention_merge(dim3 grid, hipStream_t stream, const float* partial, bf16* out, int nh, int hd, int n_splits,
-                                   long ldo) {
+                                   long ldo, const float* sink = nullptr) {
 #define GIBBS_MERGE(C)                                                                                          \
   do {                                                                                                          \
-    if (n_splits <= 4) attention_merge_kernel<C, 4><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo);      \
-    else if (n_splits <= 8) attention_merge_kernel<C, 8><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo); \
-    else attention_merge_kernel<C, 16><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo);                   \
+    if (n_splits <= 4) attention_merge_kernel<C, 4><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo, sink);      \
+    else if (n_splits <= 8) attention_merge_kernel<C, 8><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo, sink); \
+    else attention_merge_kernel<C, 16><<<grid, 256, 0, stream>>>(partial, out, nh, hd, n_splits, ldo, sink);                   \
   } while (0)
   if (hd <= WAVE) GIBBS_MERGE(1);
   else if (hd <= 2 * WAVE) GIBBS_MERGE(2);

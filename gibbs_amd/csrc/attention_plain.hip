@@ -15,7 +15,7 @@
 #include "common.h"
 
 namespace {
-constexpr int MAX_HD = 256;
+constexpr int MAX_HD = 512;
 constexpr int DPL = MAX_HD / WAVE;  // output elements per lane
 
 struct AttnArgs {
@@ -32,6 +32,7 @@ struct AttnArgs {
   int vd;               // head size of the values
   const float* bias;    // [bias_len, nh] or null: s_k += bias[min(p - k, bias_len - 1)][h]
   int bias_len;
+  const float* sink;    // [nh] or null: the softmax's denominator also holds exp(sink[h]) (no key, no value, not scaled)
 };
 
 template <typename T>
@@ -95,6 +96,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
     m = m_new;
   }
   T* o = out + (size_t)n * a.ldo + (size_t)h * vd;
+  if (a.sink) l += expf(a.sink[h] - m);
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
@@ -104,12 +106,13 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
 }
 }  // namespace
 
-// The general entry point: values of head size vd, and an optional table of score biases over the distance.
-GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
-                                               const int* pos, const int* row_req, const int* table, int max_pages,
-                                               int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
-                                               long ldq, long ldo, float scale, int window, const float* slopes,
-                                               const float* bias, int bias_len, hipStream_t stream) {
+// The general entry point: values of head size vd, an optional table of score biases over the distance, and an
+// optional sink per head (a term exp(sink[h]) in the softmax's denominator that has no key and no value).
+GIBBS_EXPORT int gibbs_attention_plain_sink(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                            const int* pos, const int* row_req, const int* table, int max_pages,
+                                            int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
+                                            long ldq, long ldo, float scale, int window, const float* slopes,
+                                            const float* bias, int bias_len, const float* sink, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "attention: bad sizes rows=%d heads=%d kv=%d hd=%d vd=%d", n_rows, nh, nkv, hd, vd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd <= MAX_HD && vd <= MAX_HD, "attention: head sizes %d, %d above %d", hd, vd, MAX_HD);
@@ -117,7 +120,7 @@ GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention: bad cache geometry");
   GIBBS_REQUIRE(!bias || bias_len > 0, "attention: an empty table of score biases");
   if (n_rows == 0) return 0;
-  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes, vd, bias, bias_len};
+  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes, vd, bias, bias_len, sink};
   dim3 grid(n_rows, ceil_div(nh, 4));
   GIBBS_REQUIRE(grid.y <= 65535, "attention: too many heads (%d)", nh);
   if (dtype == GIBBS_F32)
@@ -127,6 +130,15 @@ GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages
   else
     return gibbs_fail("attention: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("attention");
+}
+
+GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                               const int* pos, const int* row_req, const int* table, int max_pages,
+                                               int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
+                                               long ldq, long ldo, float scale, int window, const float* slopes,
+                                               const float* bias, int bias_len, hipStream_t stream) {
+  return gibbs_attention_plain_sink(q, kpages, vpages, out, dtype, pos, row_req, table, max_pages, page_size, num_pages, n_rows, nh,
+                                    nkv, hd, vd, ldq, ldo, scale, window, slopes, bias, bias_len, nullptr, stream);
 }
 
 GIBBS_EXPORT int gibbs_attention_plain(const void* q, const void* kpages, const void* vpages, void* out, int dtype,

@@ -73,6 +73,8 @@ struct PrefillArgs {
   // entry for all farther ones), divided by `scale` already (it is added to the raw scores, which are scaled later)
   const float* bias;
   int bias_len;
+  // a sink per head, or null: [nh]; the softmax's denominator also holds exp(sink[h]) (natural units, not scaled)
+  const float* sink;
 };
 
 // DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
@@ -389,6 +391,7 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
     return;
   }
   if (row < rows_here) {
+    if (a.sink) l += __expf(a.sink[head] - m * a.scale);
     const float inv = 1.0f / l;
     bf16* dst = out + (size_t)(n0 + row) * a.ldo + (size_t)head * HD + g * 4;
 #pragma unroll
@@ -431,11 +434,12 @@ void launch_prefill(dim3 grid, int heads_per_wg, hipStream_t stream, const bf16*
 // heads_per_wg: query heads of a kv head's group that a workgroup takes (1, 2 or 4; 0 counts as 1; the step's
 // rule for it is gibbs_rule_prefill_heads).
 // bias (or null): float32 [nh, bias_len], the score of a key d positions back gets bias[h][min(d, bias_len - 1)] * scale added.
-GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+// sink (or null): float32 [nh], a term exp(sink[h]) in the softmax's denominator that has no key and no value.
+GIBBS_EXPORT int gibbs_attention_prefill_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
                                               const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
                                               int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
                                               long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
-                                              const float* bias, int bias_len, hipStream_t stream) {
+                                              const float* bias, int bias_len, const float* sink, hipStream_t stream) {
   GIBBS_REQUIRE(!bias || (bias_len > 0 && scale > 0.f), "attention_prefill: an empty table of score biases, or a scale that is not positive");
   GIBBS_REQUIRE(n_rows >= 0 && n_req >= 0 && nh > 0 && nkv > 0, "attention_prefill: bad sizes rows=%d requests=%d heads=%d kv=%d", n_rows, n_req, nh, nkv);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", nh, nkv);
@@ -450,7 +454,7 @@ GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages,
                 "attention_prefill: %d heads a workgroup (1, 2 or 4 of a kv head's %d; more than one for head sizes up to 64)", heads_per_wg, nh / nkv);
   if (n_rows == 0 || n_req == 0) return 0;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits, bias, bias_len};
+  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits, bias, bias_len, sink};
   dim3 grid(ceil_div(n_rows, BM) + n_req, nh, n_splits);
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;
@@ -469,9 +473,19 @@ GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages,
     if (e != hipSuccess) return gibbs_fail("attention_prefill: %s", hipGetErrorString(e));
     dim3 mgrid(n_rows, ceil_div(nh, 4));
     launch_attention_merge(mgrid, stream, partial + (size_t)first_row * nh * n_splits * (hd + 2), oo + (size_t)first_row * ldo,
-                           nh, hd, n_splits, ldo);
+                           nh, hd, n_splits, ldo, sink);
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
+}
+
+GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                              const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
+                                              int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                              long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
+                                              const float* bias, int bias_len, hipStream_t stream) {
+  return gibbs_attention_prefill_sink(q, kpages, vpages, out, partial, cu, ctx, table, n_req, max_pages, page_size, num_pages, n_rows,
+                                      nh, nkv, hd, ldq, ldo, scale, window, n_splits, first_row, heads_per_wg, bias, bias_len, nullptr,
+                                      stream);
 }
 
 GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out, float* partial,

@@ -20,6 +20,37 @@ int gibbs_attention_plain_general(const void* q, const void* kpages, const void*
                                   const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
                                   int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window,
                                   const float* slopes, const float* bias, int bias_len, hipStream_t stream);
+int gibbs_attention_plain_sink(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
+                               const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
+                               int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window,
+                               const float* slopes, const float* bias, int bias_len, const float* sink, hipStream_t stream);
+int gibbs_attention_prefill_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                 const int* cu, const int* ctx, const int* table, int n_req, int max_pages, int page_size,
+                                 int num_pages, int n_rows, int nh, int nkv, int hd, long ldq, long ldo, float scale, int window,
+                                 int n_splits, int first_row, int heads_per_wg, const float* bias, int bias_len,
+                                 const float* sink, hipStream_t stream);
+// ---- latent.hip: what the latent-attention mixer, hyper-connected streams and their neighbours need
+int gibbs_embed_tables(const void* table, const void* pair_table, const void* pos_table, int dtype, const int* ids,
+                       const int* pos, const int* row_req, const int* cu, const int* slot, const int* prev, long slot_stride,
+                       float* x, int copies, int n, int hidden, int vocab, int buckets, int mul_prev, int mul_cur, int pos_len,
+                       hipStream_t stream);
+int gibbs_store_last_token(const int* ids, const int* cu, const int* slot, int* prev, long slot_stride, int n_req,
+                           hipStream_t stream);
+int gibbs_streams_norm(const float* x, int streams, long stream_stride, const float* coef, int kind, const float* gain,
+                       const float* bias, float eps, void* out, int dtype, const int* rows, int n_out, int hidden,
+                       hipStream_t stream);
+int gibbs_streams_write(float* x, int streams, long stream_stride, const float* mix, const float* out_coef, const void* delta,
+                        int delta_dtype, int parts, long part_stride, long count, hipStream_t stream);
+int gibbs_rms_rows_ld(const void* in, long ld_in, const float* gain, float eps, void* out, long ld_out, int dtype, int n,
+                      int width, hipStream_t stream);
+int gibbs_latent_prepare(const void* kv, long ld_kv, const void* q, long ld_q, void* q_out, long ld_qo, void* pages, int dtype,
+                         const float* gain, float eps, const float* inv_freq, int rot_dims, int variant, const int* pos,
+                         const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh,
+                         int dim, int rot, int rank, hipStream_t stream);
+int gibbs_sigmoid_gate(void* o, long ld_o, const void* g, long ld_g, int dtype, int n, int width, hipStream_t stream);
+int gibbs_poly_norm(const void* z, void* out, int dtype, const float* coef, float eps, int n, int F, hipStream_t stream);
+int gibbs_gemm_heads(const void* X, long ldx, long head_x, const void* W, long head_w, long ldw, void* Y, long ldy, long head_y,
+                     int dtype, int n, int O, int I, int heads, hipStream_t stream);
 int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype, const int* pos, const int* row_req,
                      const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
                      float eps, int unit, int norm_dim, float temp_coef, int temp_every, hipStream_t stream);

@@ -1,0 +1,473 @@
+// Kernels of the latent-attention mixer and of its neighbours in a model: an embedding that adds rows of a
+// hashed token-pair table and of a learned position table, several residual streams that a layer reads as
+// one weighted sum and writes through a small mixing matrix (hyper-connections), layer norm, the rotation
+// of a latent attention's shared key part, an output gate, and the polynomial-norm activation.
+//
+// Sums, norms, angles and the streams themselves are float32 whatever the run's activation type is.
+#include "common.h"
+
+namespace {
+// ------------------------------------------------------------------------------------------------- embedding
+// x[c][n][:] = table[id] + pair_table[row] + pos_table[pos], c = 0 .. copies - 1, with
+//   row = buckets                                  for a sequence's first token (position 0)
+//         (prev * mul_prev + id * mul_cur) mod buckets   otherwise,
+// prev being the row before in this step, or, for the first row of a request's portion, the token that the
+// request's state slot holds (what gibbs_store_last_token left there).
+template <typename T>
+__global__ void embed_tables_kernel(const T* __restrict__ table, const T* __restrict__ pair_table, const T* __restrict__ pos_table,
+                                    const int* __restrict__ ids, const int* __restrict__ pos, const int* __restrict__ row_req,
+                                    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ prev,
+                                    long slot_stride, float* __restrict__ x, int copies, int n_rows, int hidden, int vocab,
+                                    int buckets, int mul_prev, int mul_cur, int pos_len) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);      // (never read outside the table)
+  const T* row = table + (size_t)id * hidden;
+  const T* pair = nullptr;
+  const int p = pos[n];
+  if (pair_table) {
+    long r = buckets;
+    if (p > 0) {
+      const int req = row_req[n];
+      int before = n > cu[req] ? ids[n - 1] : prev[(size_t)slot[req] * slot_stride];
+      before = before < 0 ? 0 : (before >= vocab ? vocab - 1 : before);
+      r = ((long)before * mul_prev + (long)id * mul_cur) % buckets;
+    }
+    pair = pair_table + (size_t)r * hidden;
+  }
+  const T* at = pos_table ? pos_table + (size_t)min(max(p, 0), pos_len - 1) * hidden : nullptr;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = to_float(row[i]);
+    if (pair) v += to_float(pair[i]);
+    if (at) v += to_float(at[i]);
+    for (int c = 0; c < copies; ++c) x[((size_t)c * n_rows + n) * hidden + i] = v;
+  }
+}
+
+__global__ void store_last_token_kernel(const int* __restrict__ ids, const int* __restrict__ cu, const int* __restrict__ slot,
+                                        int* __restrict__ prev, long slot_stride, int n_req) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_req || cu[r + 1] <= cu[r]) return;
+  prev[(size_t)slot[r] * slot_stride] = ids[cu[r + 1] - 1];
+}
+
+// ------------------------------------------------------------------------------------------------- streams
+// out[j][:] = norm(u), u = sum_s coef[s] x[s][row j][:] (coef null: every stream counts 1), s ascending.
+// kind 0: u / sqrt(mean(u^2) + eps) * gain;  kind 1: (u - mean) / sqrt(mean((u - mean)^2) + eps) * gain + bias.
+// gain or bias null: 1 and 0.  One workgroup per row; u is kept in LDS (hidden floats).
+template <typename T>
+__global__ void streams_norm_kernel(const float* __restrict__ x, int streams, long stream_stride, const float* __restrict__ coef,
+                                    int kind, const float* __restrict__ gain, const float* __restrict__ bias, float eps,
+                                    T* __restrict__ out, const int* __restrict__ rows, int hidden) {
+  extern __shared__ float u[];
+  __shared__ float scratch[16];
+  const int j = blockIdx.x;
+  const size_t row = rows ? rows[j] : j;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = 0.f;
+    for (int s = 0; s < streams; ++s) {
+      const float xs = x[(size_t)s * stream_stride + row * hidden + i];
+      v = coef ? fmaf(coef[s], xs, v) : v + xs;
+    }
+    u[i] = v;
+    sum += v;
+  }
+  float mean = 0.f;
+  if (kind == 1) mean = block_sum(sum, scratch) / (float)hidden;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float d = u[i] - mean;
+    sq = fmaf(d, d, sq);
+  }
+  const float r = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = (u[i] - mean) * r;
+    if (gain) v *= gain[i];
+    if (bias && kind == 1) v += bias[i];
+    out[(size_t)j * hidden + i] = from_float<T>(v);
+  }
+}
+
+// All streams at once from the old ones: x[t] <- sum_s mix[s][t] x[s] + out_coef[t] * y, s ascending, where y is
+// the delta (one part in the activation type, or float32 partial sums added in ascending order).
+template <int S, typename T>
+__global__ void streams_write_kernel(float* __restrict__ x, long stream_stride, const float* __restrict__ mix,
+                                     const float* __restrict__ out_coef, const T* __restrict__ delta, int parts, long part_stride,
+                                     long count) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float y = 0.f;
+  for (int p = 0; p < parts; ++p) y += to_float(delta[(size_t)p * part_stride + i]);
+  float old[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) old[s] = x[(size_t)s * stream_stride + i];
+#pragma unroll
+  for (int t = 0; t < S; ++t) {
+    float v = 0.f;
+#pragma unroll
+    for (int s = 0; s < S; ++s) v = fmaf(mix[s * S + t], old[s], v);
+    x[(size_t)t * stream_stride + i] = fmaf(out_coef[t], y, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------- rows
+// out[n][:] = in[n][:width] / sqrt(mean(in^2) + eps) * gain; one wave per row.
+template <typename T>
+__global__ void rms_rows_ld_kernel(const T* __restrict__ in, long ld_in, const float* __restrict__ gain, float eps,
+                                   T* __restrict__ out, long ld_out, int n, int width) {
+  const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (row >= n) return;
+  const T* src = in + (size_t)row * ld_in;
+  float sq = 0.f;
+  for (int i = lane; i < width; i += WAVE) {
+    const float v = to_float(src[i]);
+    sq = fmaf(v, v, sq);
+  }
+  const float r = 1.0f / sqrtf(wave_sum(sq) / (float)width + eps);
+  for (int i = lane; i < width; i += WAVE) out[(size_t)row * ld_out + i] = from_float<T>(to_float(src[i]) * r * (gain ? gain[i] : 1.f));
+}
+
+// The pair (u, v) at position p becomes (u cos a - v sin a, v cos a + u sin a), a = float(p) * inv_freq[i].
+// variant 0: pairs (i, i + dims / 2); 1: pairs (2 i, 2 i + 1); entries from `dims` on pass unchanged.
+template <typename T>
+__device__ __forceinline__ void rotate_into(const T* __restrict__ src, T* __restrict__ dst, int width, int dims, int variant,
+                                            const float* __restrict__ inv_freq, float p, int lane, int lanes) {
+  const int half = dims / 2;
+  for (int i = lane; i < half; i += lanes) {
+    const int a = variant ? 2 * i : i, b = variant ? 2 * i + 1 : i + half;
+    const float angle = p * inv_freq[i];
+    const float c = cosf(angle), s = sinf(angle);
+    const float u = to_float(src[a]), v = to_float(src[b]);
+    dst[a] = from_float<T>(u * c - v * s);
+    dst[b] = from_float<T>(v * c + u * s);
+  }
+  for (int i = dims + lane; i < width; i += lanes) dst[i] = src[i];
+}
+
+// What a latent attention does to a step's rows before the scores: per row n at position p of request r,
+//   the cached row  page[p] = [ kv[n][:rank] / rms * gain | rotate(kv[n][rank : rank + rot]) ]   (one per token, shared by all heads)
+//   the queries' rotated parts  q_out[n][h][rank : rank + rot] = rotate(q[n][h][dim : dim + rot]).
+// (The queries' first `rank` entries, their unrotated parts taken through the keys' up-projection, are another kernel's.)
+// One workgroup of 64 threads per (row, y): y = 0 the cached row, y = 1 .. the heads in groups of 4.
+template <typename T>
+__global__ void latent_prepare_kernel(const T* __restrict__ kv, long ld_kv, const T* __restrict__ q, long ld_q, T* __restrict__ q_out,
+                                      long ld_qo, T* __restrict__ pages, const float* __restrict__ gain, float eps,
+                                      const float* __restrict__ inv_freq, int dims, int variant, const int* __restrict__ pos,
+                                      const int* __restrict__ row_req, const int* __restrict__ table, int max_pages, int page_size,
+                                      int num_pages, int nh, int dim, int rot, int rank) {
+  const int n = blockIdx.x, lane = threadIdx.x;
+  const int p = pos[n];
+  if (blockIdx.y == 0) {
+    int page = table[(size_t)row_req[n] * max_pages + p / page_size];
+    page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);      // never write outside the pool
+    T* dst = pages + ((size_t)page * page_size + p % page_size) * (rank + rot);
+    const T* src = kv + (size_t)n * ld_kv;
+    float sq = 0.f;
+    for (int i = lane; i < rank; i += WAVE) {
+      const float v = to_float(src[i]);
+      sq = fmaf(v, v, sq);
+    }
+    const float r = 1.0f / sqrtf(wave_sum(sq) / (float)rank + eps);
+    for (int i = lane; i < rank; i += WAVE) dst[i] = from_float<T>(to_float(src[i]) * r * (gain ? gain[i] : 1.f));
+    rotate_into(src + rank, dst + rank, rot, dims, variant, inv_freq, (float)p, lane, WAVE);
+    return;
+  }
+  for (int h = (blockIdx.y - 1) * 4; h < min(nh, (int)blockIdx.y * 4); ++h)
+    rotate_into(q + (size_t)n * ld_q + (size_t)h * (dim + rot) + dim, q_out + (size_t)n * ld_qo + (size_t)h * (rank + rot) + rank, rot,
+                dims, variant, inv_freq, (float)p, lane, WAVE);
+}
+
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ o, long ld_o, const T* __restrict__ g, long ld_g, int n, int width) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)n * width) return;
+  const long row = i / width, col = i % width;
+  const float z = to_float(g[row * ld_g + col]);
+  T* at = o + row * ld_o + col;
+  *at = from_float<T>(to_float(*at) / (1.0f + expf(-z)));
+}
+
+// out = a N(z) + b N(z^2) + c N(z^3) + e over a row of F values, N(v) = v / sqrt(mean(v^2) + eps), powers element by element.
+template <typename T>
+__global__ void poly_norm_kernel(const T* __restrict__ z, T* __restrict__ out, const float* __restrict__ coef, float eps, int F) {
+  __shared__ float scratch[16];
+  const T* src = z + (size_t)blockIdx.x * F;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+    const float v = to_float(src[i]), v2 = v * v;
+    s2 += v2;
+    s4 = fmaf(v2, v2, s4);
+    s6 = fmaf(v2 * v, v2 * v, s6);
+  }
+  const float r1 = coef[0] / sqrtf(block_sum(s2, scratch) / (float)F + eps);
+  const float r2 = coef[1] / sqrtf(block_sum(s4, scratch) / (float)F + eps);
+  const float r3 = coef[2] / sqrtf(block_sum(s6, scratch) / (float)F + eps);
+  const float e = coef[3];
+  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+    const float v = to_float(src[i]), v2 = v * v;
+    out[(size_t)blockIdx.x * F + i] = from_float<T>(fmaf(r1, v, fmaf(r2, v2, fmaf(r3, v2 * v, e))));
+  }
+}
+
+// ------------------------------------------------------------------------------------------------- per-head products
+// Y[n][h][o] = sum_k X[n][h][k] W[h][o][k] for every head h: a product per head over slices of the same rows
+// (X + h * head_x, row stride ldx; W + h * head_w, row stride ldw; Y + h * head_y, row stride ldy).
+// Plain FMA, every element in ascending k: the 32-bit path, and bfloat16 slices that are not 16-byte aligned.
+constexpr int TM = 64, TN = 64, TK = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_heads_plain_kernel(const T* __restrict__ X, long ldx, long head_x, const T* __restrict__ W,
+                                                               long head_w, long ldw, T* __restrict__ Y, long ldy, long head_y, int N,
+                                                               int O, int I) {
+  __shared__ float sa[TK][TM + 4];
+  __shared__ float sw[TK][TN + 4];
+  const int h = blockIdx.z;
+  X += (size_t)h * head_x;
+  W += (size_t)h * head_w;
+  Y += (size_t)h * head_y;
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  const int row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < I; k0 += TK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = threadIdx.x + i * 256;
+      const int r = e / TK, k = e % TK;
+      const int gr = row0 + r, gc = col0 + r, gk = k0 + k;
+      sa[k][r] = (gr < N && gk < I) ? to_float(X[(size_t)gr * ldx + gk]) : 0.f;
+      sw[k][r] = (gc < O && gk < I) ? to_float(W[(size_t)gc * ldw + gk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TK; ++k) {
+      float a[4], w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = sa[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = sw[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gr = row0 + ty * 4 + i;
+    if (gr >= N) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gc = col0 + tx * 4 + j;
+      if (gc < O) Y[(size_t)gr * ldy + gc] = from_float<T>(acc[i][j]);
+    }
+  }
+}
+
+// The same on the matrix cores, for bfloat16 slices whose rows start at multiples of 16 bytes and whose inner
+// size is a multiple of 8: a wave takes 16 rows x 64 features, four 16 x 16 x 32 products per step of k, both
+// operands straight from memory (X and W are contiguous along k, which is the operand layout: lane l holds
+// the 8 values k = (l / 16) * 8 .. + 8 of row or feature l % 16); a workgroup is 4 waves on 64 rows.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+__global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(const bf16* __restrict__ X, long ldx, long head_x, const bf16* __restrict__ W,
+                                                              long head_w, long ldw, bf16* __restrict__ Y, long ldy, long head_y, int N,
+                                                              int O, int I) {
+  const int h = blockIdx.z;
+  X += (size_t)h * head_x;
+  W += (size_t)h * head_w;
+  Y += (size_t)h * head_y;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int lr = lane % 16, lg = lane / 16;
+  const int row = blockIdx.y * 64 + wave * 16 + lr;
+  const int col0 = blockIdx.x * 64;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  floatx4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const bf16* xr = X + (size_t)min(row, N - 1) * ldx;
+  for (int k0 = 0; k0 < I; k0 += 32) {
+    const int k = k0 + lg * 8;
+    const bf16x8 a = (row < N && k < I) ? *(const bf16x8*)(xr + k) : zero8;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int col = col0 + t * 16 + lr;
+      const bf16x8 b = (col < O && k < I) ? *(const bf16x8*)(W + (size_t)col * ldw + k) : zero8;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+    }
+  }
+  // element i of a lane's result: row (lane / 16) * 4 + i of the wave's 16, feature lane % 16 of the tile
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int col = col0 + t * 16 + lr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = blockIdx.y * 64 + wave * 16 + lg * 4 + i;
+      if (r < N && col < O) Y[(size_t)r * ldy + col] = (bf16)acc[t][i];
+    }
+  }
+}
+}  // namespace
+
+GIBBS_EXPORT int gibbs_embed_tables(const void* table, const void* pair_table, const void* pos_table, int dtype, const int* ids,
+                                    const int* pos, const int* row_req, const int* cu, const int* slot, const int* prev,
+                                    long slot_stride, float* x, int copies, int n, int hidden, int vocab, int buckets, int mul_prev,
+                                    int mul_cur, int pos_len, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && hidden > 0 && vocab > 0 && copies >= 1, "embed_tables: bad sizes n=%d hidden=%d vocab=%d copies=%d", n, hidden, vocab, copies);
+  GIBBS_REQUIRE(table && ids && pos && x, "embed_tables: the table, ids, positions and rows are needed");
+  GIBBS_REQUIRE(!pair_table || (buckets > 0 && row_req && cu && slot && prev), "embed_tables: the pair table needs its buckets, the batch's layout and the requests' last tokens");
+  GIBBS_REQUIRE(!pos_table || pos_len > 0, "embed_tables: an empty position table");
+  if (n == 0) return 0;
+  const int threads = hidden >= 1024 ? 256 : 64;
+  if (dtype == GIBBS_F32)
+    embed_tables_kernel<float><<<n, threads, 0, stream>>>((const float*)table, (const float*)pair_table, (const float*)pos_table, ids, pos,
+                                                          row_req, cu, slot, prev, slot_stride, x, copies, n, hidden, vocab, buckets,
+                                                          mul_prev, mul_cur, pos_len);
+  else if (dtype == GIBBS_BF16)
+    embed_tables_kernel<bf16><<<n, threads, 0, stream>>>((const bf16*)table, (const bf16*)pair_table, (const bf16*)pos_table, ids, pos,
+                                                         row_req, cu, slot, prev, slot_stride, x, copies, n, hidden, vocab, buckets,
+                                                         mul_prev, mul_cur, pos_len);
+  else
+    return gibbs_fail("embed_tables: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("embed_tables");
+}
+
+// prev[slot[r] * slot_stride] = the last token of request r's rows in this step (after the embedding has read what was there).
+GIBBS_EXPORT int gibbs_store_last_token(const int* ids, const int* cu, const int* slot, int* prev, long slot_stride, int n_req,
+                                        hipStream_t stream) {
+  GIBBS_REQUIRE(n_req >= 0 && ids && cu && slot && prev, "store_last_token: missing operands");
+  if (n_req == 0) return 0;
+  store_last_token_kernel<<<ceil_div(n_req, 64), 64, 0, stream>>>(ids, cu, slot, prev, slot_stride, n_req);
+  GIBBS_LAUNCH_STATUS("store_last_token");
+}
+
+GIBBS_EXPORT int gibbs_streams_norm(const float* x, int streams, long stream_stride, const float* coef, int kind, const float* gain,
+                                    const float* bias, float eps, void* out, int dtype, const int* rows, int n_out, int hidden,
+                                    hipStream_t stream) {
+  GIBBS_REQUIRE(n_out >= 0 && hidden > 0 && streams >= 1 && (kind == 0 || kind == 1), "streams_norm: bad sizes rows=%d hidden=%d streams=%d kind=%d", n_out, hidden, streams, kind);
+  GIBBS_REQUIRE(hidden <= 16000, "streams_norm: rows of %d values do not fit the workgroup's memory", hidden);
+  if (n_out == 0) return 0;
+  const int threads = hidden >= 2048 ? 256 : (hidden >= 512 ? 128 : 64);
+  const size_t lds = (size_t)hidden * 4;
+  if (dtype == GIBBS_F32)
+    streams_norm_kernel<float><<<n_out, threads, lds, stream>>>(x, streams, stream_stride, coef, kind, gain, bias, eps, (float*)out, rows, hidden);
+  else if (dtype == GIBBS_BF16)
+    streams_norm_kernel<bf16><<<n_out, threads, lds, stream>>>(x, streams, stream_stride, coef, kind, gain, bias, eps, (bf16*)out, rows, hidden);
+  else
+    return gibbs_fail("streams_norm: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("streams_norm");
+}
+
+template <typename T>
+static int launch_streams_write(float* x, int streams, long stream_stride, const float* mix, const float* out_coef, const T* delta,
+                                int parts, long part_stride, long count, hipStream_t stream) {
+  const int blocks = ceil_div(count, 256);
+  switch (streams) {
+#define GIBBS_STREAMS(S) \
+  case S: streams_write_kernel<S, T><<<blocks, 256, 0, stream>>>(x, stream_stride, mix, out_coef, delta, parts, part_stride, count); break;
+    GIBBS_STREAMS(1) GIBBS_STREAMS(2) GIBBS_STREAMS(3) GIBBS_STREAMS(4) GIBBS_STREAMS(5) GIBBS_STREAMS(6) GIBBS_STREAMS(7) GIBBS_STREAMS(8)
+#undef GIBBS_STREAMS
+    default: return gibbs_fail("streams_write: %d streams (1 to 8)", streams);
+  }
+  GIBBS_LAUNCH_STATUS("streams_write");
+}
+// delta: [count] in delta_dtype (parts 1), or float32 partial sums [parts, count] (part_stride apart).
+GIBBS_EXPORT int gibbs_streams_write(float* x, int streams, long stream_stride, const float* mix, const float* out_coef,
+                                     const void* delta, int delta_dtype, int parts, long part_stride, long count, hipStream_t stream) {
+  GIBBS_REQUIRE(count >= 0 && parts >= 1 && x && mix && out_coef && delta, "streams_write: missing operands");
+  GIBBS_REQUIRE(parts == 1 || delta_dtype == GIBBS_F32, "streams_write: partial sums are float32");
+  if (count == 0) return 0;
+  if (delta_dtype == GIBBS_F32) return launch_streams_write(x, streams, stream_stride, mix, out_coef, (const float*)delta, parts, part_stride, count, stream);
+  if (delta_dtype == GIBBS_BF16) return launch_streams_write(x, streams, stream_stride, mix, out_coef, (const bf16*)delta, parts, part_stride, count, stream);
+  return gibbs_fail("streams_write: unknown dtype %d", delta_dtype);
+}
+
+GIBBS_EXPORT int gibbs_rms_rows_ld(const void* in, long ld_in, const float* gain, float eps, void* out, long ld_out, int dtype, int n,
+                                   int width, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && width > 0 && ld_in >= width && ld_out >= width, "rms_rows: bad sizes n=%d width=%d", n, width);
+  if (n == 0) return 0;
+  if (dtype == GIBBS_F32)
+    rms_rows_ld_kernel<float><<<ceil_div(n, 4), 256, 0, stream>>>((const float*)in, ld_in, gain, eps, (float*)out, ld_out, n, width);
+  else if (dtype == GIBBS_BF16)
+    rms_rows_ld_kernel<bf16><<<ceil_div(n, 4), 256, 0, stream>>>((const bf16*)in, ld_in, gain, eps, (bf16*)out, ld_out, n, width);
+  else
+    return gibbs_fail("rms_rows: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("rms_rows");
+}
+
+// kv: rows [n, >= rank + rot] (the down-projection's result); q: rows of nh heads of dim + rot; q_out: rows of nh heads of
+// rank + rot, of which this call fills the last rot; pages: [num_pages, page_size, rank + rot] of one layer.
+GIBBS_EXPORT int gibbs_latent_prepare(const void* kv, long ld_kv, const void* q, long ld_q, void* q_out, long ld_qo, void* pages,
+                                      int dtype, const float* gain, float eps, const float* inv_freq, int rot_dims, int variant,
+                                      const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
+                                      int num_pages, int n_rows, int nh, int dim, int rot, int rank, hipStream_t stream) {
+  GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && dim >= 0 && rot >= 0 && rank > 0, "latent_prepare: bad sizes rows=%d heads=%d dim=%d rot=%d rank=%d", n_rows, nh, dim, rot, rank);
+  GIBBS_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq), "latent_prepare: %d rotated dimensions of %d", rot_dims, rot);
+  GIBBS_REQUIRE(variant == 0 || variant == 1, "latent_prepare: unknown pairing %d", variant);
+  GIBBS_REQUIRE(ld_kv >= rank + rot && ld_q >= (long)nh * (dim + rot) && ld_qo >= (long)nh * (rank + rot), "latent_prepare: row strides shorter than rows");
+  GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0, "latent_prepare: bad cache geometry");
+  if (n_rows == 0) return 0;
+  dim3 grid(n_rows, 1 + ceil_div(nh, 4));
+  GIBBS_REQUIRE(grid.y <= 65535, "latent_prepare: too many heads (%d)", nh);
+  if (dtype == GIBBS_F32)
+    latent_prepare_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)kv, ld_kv, (const float*)q, ld_q, (float*)q_out, ld_qo, (float*)pages,
+                                                            gain, eps, inv_freq, rot_dims, variant, pos, row_req, table, max_pages, page_size,
+                                                            num_pages, nh, dim, rot, rank);
+  else if (dtype == GIBBS_BF16)
+    latent_prepare_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)kv, ld_kv, (const bf16*)q, ld_q, (bf16*)q_out, ld_qo, (bf16*)pages,
+                                                           gain, eps, inv_freq, rot_dims, variant, pos, row_req, table, max_pages, page_size,
+                                                           num_pages, nh, dim, rot, rank);
+  else
+    return gibbs_fail("latent_prepare: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("latent_prepare");
+}
+
+// o[n][:width] *= sigmoid(g[n][:width]), in place.
+GIBBS_EXPORT int gibbs_sigmoid_gate(void* o, long ld_o, const void* g, long ld_g, int dtype, int n, int width, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && width > 0 && ld_o >= width && ld_g >= width, "sigmoid_gate: bad sizes n=%d width=%d", n, width);
+  if (n == 0) return 0;
+  const int blocks = ceil_div((long)n * width, 256);
+  if (dtype == GIBBS_F32)
+    sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)o, ld_o, (const float*)g, ld_g, n, width);
+  else if (dtype == GIBBS_BF16)
+    sigmoid_gate_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)o, ld_o, (const bf16*)g, ld_g, n, width);
+  else
+    return gibbs_fail("sigmoid_gate: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("sigmoid_gate");
+}
+
+// coef: float32 [4] on the device: a, b, c, e.
+GIBBS_EXPORT int gibbs_poly_norm(const void* z, void* out, int dtype, const float* coef, float eps, int n, int F, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && F > 0 && coef, "poly_norm: bad sizes n=%d F=%d", n, F);
+  if (n == 0) return 0;
+  const int threads = F >= 2048 ? 256 : (F >= 512 ? 128 : 64);
+  if (dtype == GIBBS_F32)
+    poly_norm_kernel<float><<<n, threads, 0, stream>>>((const float*)z, (float*)out, coef, eps, F);
+  else if (dtype == GIBBS_BF16)
+    poly_norm_kernel<bf16><<<n, threads, 0, stream>>>((const bf16*)z, (bf16*)out, coef, eps, F);
+  else
+    return gibbs_fail("poly_norm: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("poly_norm");
+}
+
+GIBBS_EXPORT int gibbs_gemm_heads(const void* X, long ldx, long head_x, const void* W, long head_w, long ldw, void* Y, long ldy,
+                                  long head_y, int dtype, int n, int O, int I, int heads, hipStream_t stream) {
+  GIBBS_REQUIRE(n >= 0 && O > 0 && I > 0 && heads > 0 && heads <= 65535, "gemm_heads: bad sizes n=%d O=%d I=%d heads=%d", n, O, I, heads);
+  GIBBS_REQUIRE(ldx >= I && ldw >= I && ldy >= O, "gemm_heads: row strides shorter than rows");
+  if (n == 0) return 0;
+  dim3 grid(ceil_div(O, 64), ceil_div(n, 64), heads);
+  GIBBS_REQUIRE(grid.y <= 65535, "gemm_heads: too many rows (%d)", n);
+  if (dtype == GIBBS_F32) {
+    gemm_heads_plain_kernel<float><<<grid, 256, 0, stream>>>((const float*)X, ldx, head_x, (const float*)W, head_w, ldw, (float*)Y, ldy, head_y, n, O, I);
+  } else if (dtype == GIBBS_BF16) {
+    const bool aligned = I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && head_x % 8 == 0 && head_w % 8 == 0 && ((uintptr_t)X % 16) == 0 &&
+                         ((uintptr_t)W % 16) == 0;
+    if (aligned)
+      gemm_heads_mfma_kernel<<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I);
+    else
+      gemm_heads_plain_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I);
+  } else {
+    return gibbs_fail("gemm_heads: unknown dtype %d", dtype);
+  }
+  GIBBS_LAUNCH_STATUS("gemm_heads");
+}

@@ -264,6 +264,9 @@ struct NormPart {
   virtual Pending run_on(Exec& e, Pending delta) const;
   // x += norm(a part's result) in one pass, where the norm can (else: false, and nothing is done)
   virtual bool add_normed(Exec& e, float* x, Pending delta) const { return false; }
+  // the norm of a weighted sum of several residual streams x [streams][N][hidden] (coef null: their plain sum), of all
+  // rows or of `rows`; the streams are not touched
+  virtual void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const;
 };
 
 struct Body {
@@ -276,14 +279,35 @@ struct Body {
   virtual int cache_group() const { return -1; }
 };
 
+// How a sublayer reads and writes several residual streams (hyper-connections): it reads u = sum_s in[s] x_s, and
+// writes x_t <- sum_s mix[s][t] x_s + out[t] y for all t at once.
+struct Hyper {
+  const float* in = nullptr;    // [streams]
+  const float* mix = nullptr;   // [streams, streams], indexed [from][to]
+  const float* out = nullptr;   // [streams]
+};
+
 struct Plan {
   int dtype = GIBBS_BF16;   // activations, matrices and cache pages
   int hidden = 0, vocab = 0;
   const void* table = nullptr;
   int table_dtype = GIBBS_BF16;
+  // residual streams: x is [streams][rows][hidden], every stream starting as the embedding's output
+  int streams = 1;
+  std::vector<Hyper> hypers;
+  // tables whose rows are added to the token table's: one over hashed pairs (previous token, token), the row
+  // `buckets` for a sequence's first token, and one over positions; the previous token of a request lives in its
+  // state slot (prev_state [slots] int32, slot_stride words apart)
+  const void* pair_table = nullptr;
+  int buckets = 0, mul_prev = 0, mul_cur = 0;
+  const void* pos_table = nullptr;
+  int pos_len = 0;
+  int* prev_state = nullptr;
+  long prev_stride = 0;
+  bool table_sums() const { return pair_table || pos_table || streams > 1; }
   float embed_scale = 1.0f;            // the table's rows are multiplied by it
   const float* embed_inv_freq = nullptr;   // [hidden / 2]: a sinusoidal position vector is added to the rows
-  bool plain_embedding() const { return embed_scale == 1.0f && !embed_inv_freq && !reinjects; }
+  bool plain_embedding() const { return embed_scale == 1.0f && !embed_inv_freq && !reinjects && !table_sums(); }
   bool reinjects = false;              // the program adds the embedding's output into the stream again
   Matrix head;
   int tail = -1;            // the norm in front of the head
@@ -291,7 +315,7 @@ struct Plan {
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
   std::vector<std::unique_ptr<NormPart>> norms;
   std::vector<std::unique_ptr<Body>> bodies;
-  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT, OP_ADD_NORMED };
+  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT, OP_ADD_NORMED, OP_STREAMS_NORM, OP_STREAMS_ADD };
   struct Op {
     int kind, norm, body, value;   // value: what a body reads, an add adds, a drop drops
     int result;                    // the value that a norm or a body makes
@@ -301,6 +325,7 @@ struct Plan {
   mutable int last_fused = 0;
   bool has_norm(int i) const { return i >= 0 && i < (int)norms.size(); }
   bool has_body(int i) const { return i >= 0 && i < (int)bodies.size(); }
+  bool has_hyper(int i) const { return i >= 0 && i < (int)hypers.size(); }
 };
 
 Exec::Exec(const Plan& plan, const GibbsStepArgs& args)
@@ -353,9 +378,19 @@ Pending NormPart::run_on(Exec& e, Pending delta) const {
   if (!e.status) e.status = gibbs_fail("step: this norm cannot be applied to a part's result");
   return delta;
 }
+void* NormPart::run_streams(Exec& e, const float*, int, const float*, const int*, int) const {
+  if (!e.status) e.status = gibbs_fail("step: this norm cannot read several residual streams");
+  return nullptr;
+}
 struct RmsNorm : NormPart {
   const float* gain = nullptr;   // null: folded into the matrices that follow
   float eps = 0.f;
+  void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const override {
+    const int H = e.p.hidden;
+    void* out = e.take((long)n_out * H * e.esize);
+    RUN(e, gibbs_streams_norm(x, streams, (long)e.a.n_rows * H, coef, 0, gain, nullptr, eps, out, e.p.dtype, rows, n_out, H, e.a.stream));
+    return out;
+  }
   void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const override {
     const int H = e.p.hidden;
     void* out = e.take((long)n_out * H * e.esize);
@@ -384,6 +419,22 @@ struct RmsNorm : NormPart {
     RUN(e, gibbs_rmsnorm_rows(delta.data, std::max(delta.parts, 1), (long)N * H, gain, eps, out.data, e.p.dtype, N, H, e.a.stream));
     e.give(delta.data);
     return out;
+  }
+};
+// Layer norm with gain and bias: (x - mean) / sqrt(mean((x - mean)^2) + eps) * gain + bias, all in float32.
+struct LayerNorm : NormPart {
+  const float* gain = nullptr;
+  const float* bias = nullptr;
+  float eps = 0.f;
+  void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const override {
+    const int H = e.p.hidden;
+    void* out = e.take((long)n_out * H * e.esize);
+    RUN(e, gibbs_streams_norm(x, streams, (long)e.a.n_rows * H, coef, 1, gain, bias, eps, out, e.p.dtype, rows, n_out, H, e.a.stream));
+    return out;
+  }
+  void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const override {
+    e.settle(x, pending);
+    return run_streams(e, x, 1, nullptr, rows, n_out);
   }
 };
 struct HostNorm : NormPart {
@@ -437,6 +488,64 @@ struct ConvBody : Body {
 };
 
 // ---- attention over the paged cache
+// What the attention kernels need to know of a mixer whose rows are prepared (normed, rotated, the new keys and
+// values in their pages): q [N, nh * hd] (row stride ldq) against keys of head size hd and values of head size vd.
+struct PagedAttention {
+  void* kpages;
+  void* vpages;
+  int num_pages, page_size, group;
+  int nh, nkv, hd, vd;
+  float scale;
+  int window;
+  const float* slopes;    // a bias on the scores by distance: the plain kernel takes it
+  const float* bias;      // [bias_len, nh]
+  const float* bias_t;    // the same as [nh, bias_len] divided by the scale: what the matrix-core kernels add to raw scores
+  int bias_len;
+  const float* sink;      // [nh]: a term exp(sink[h]) in the softmax's denominator without key or value
+};
+void decode_attention(Exec& e, const PagedAttention& t, const void* q, long ldq, int n_rows, const int* pos, const int* row_req, void* o) {
+  int n_splits, waves;
+  decode_splits(n_rows, t.nkv, t.nh / t.nkv, e.a.max_seq, t.hd, t.page_size, 0, &n_splits, &waves);
+  float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(n_rows, t.nh, t.hd, n_splits) * 4) : nullptr;
+  RUN(e, gibbs_attention_decode_sink(q, t.kpages, t.vpages, o, partial, pos, row_req, e.table(t.group), e.width(t.group), t.page_size,
+                                     t.num_pages, n_rows, t.nh, t.nkv, t.hd, ldq, (long)t.nh * t.hd, t.scale, t.window, n_splits, waves, 0,
+                                     e.a.max_seq, t.bias_t, t.bias_len, t.sink, e.a.stream));
+  e.give(partial);
+}
+// attention of prepared rows, whatever the step's rows are; returns [N, nh * vd] (row stride ldo)
+void* attend_prepared(Exec& e, const PagedAttention& t, void* raw, long ldq, long ldo) {
+  const GibbsStepArgs& a = e.a;
+  const int N = a.n_rows;
+  const int* table = e.table(t.group);
+  const int width = e.width(t.group);
+  void* att = e.take((long)N * ldo * e.esize);
+  // the matrix-core kernels take rows that are prepared (whatever prepared them), keys and values of one head
+  // size, and a bias on the scores as a table over the distance (no slopes)
+  const bool matrix_sizes = t.hd % 16 == 0 && t.hd <= 128;
+  const bool fast_bf16 = e.bf16_run && !t.slopes && t.vd == t.hd && (!t.bias || (t.bias_t && matrix_sizes)) && (!t.sink || t.scale > 0.f);
+  if (fast_bf16 && a.max_q > 1 && matrix_sizes) {
+    // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
+    // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
+    // matrix-core kernel
+    const int lead = a.lead_single >= 2 ? a.lead_single : 0;
+    if (lead) decode_attention(e, t, raw, ldq, lead, a.pos, a.row_req, att);
+    const int rows = N - lead, reqs = a.n_req - lead;
+    const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), t.nh, a.max_seq, t.window) : 1;
+    float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(N, t.nh, t.hd, n_splits) * 4) : nullptr;
+    RUN(e, gibbs_attention_prefill_sink(raw, t.kpages, t.vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
+                                        width, t.page_size, t.num_pages, rows, t.nh, t.nkv, t.hd, ldq, ldo, t.scale, t.window, n_splits, lead,
+                                        prefill_heads(rows, reqs, t.nh, t.nkv, t.hd, a.max_seq, n_splits), t.bias_t, t.bias_len, t.sink,
+                                        a.stream));
+    e.give(partial);
+  } else if (fast_bf16 && a.max_q == 1 && t.hd % 8 == 0 && t.hd <= 256 && (!t.bias || matrix_sizes)) {
+    decode_attention(e, t, raw, ldq, N, a.pos, a.row_req, att);
+  } else {
+    RUN(e, gibbs_attention_plain_sink(raw, t.kpages, t.vpages, att, e.p.dtype, a.pos, a.row_req, table, width, t.page_size, t.num_pages,
+                                      N, t.nh, t.nkv, t.hd, t.vd, ldq, ldo, t.scale, t.window, t.slopes, t.bias, t.bias_len, t.sink, a.stream));
+  }
+  return att;
+}
+
 struct AttnBody : Body {
   Matrix qkv, out;
   const void* qkv_packed = nullptr;   // for the fused kernel
@@ -492,14 +601,8 @@ struct AttnBody : Body {
     e.skinny_residual(att, out, x, mirror);
     e.give(att);
   }
-  void decode_attention(Exec& e, const void* q, long ldq, int n_rows, const int* pos, const int* row_req, void* o) const {
-    int n_splits, waves;
-    decode_splits(n_rows, nkv, nh / nkv, e.a.max_seq, hd, page_size, 0, &n_splits, &waves);
-    float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(n_rows, nh, hd, n_splits) * 4) : nullptr;
-    RUN(e, gibbs_attention_decode_bias(q, kpages, vpages, o, partial, pos, row_req, e.table(group), e.width(group), page_size, num_pages,
-                                       n_rows, nh, nkv, hd, ldq, (long)nh * hd, scale, window, n_splits, waves, 0, e.a.max_seq, bias_t,
-                                       bias_len, e.a.stream));
-    e.give(partial);
+  PagedAttention paged() const {
+    return PagedAttention{kpages, vpages, num_pages, page_size, group, nh, nkv, hd, vd, scale, window, slopes, bias, bias_t, bias_len, nullptr};
   }
   // q/k norm, rotation and the cache write of the step's rows (a mixer that reads another's cache writes nothing)
   void prepare_rows(Exec& e, void* raw, long ldq) const {
@@ -541,32 +644,7 @@ struct AttnBody : Body {
       att = attend_decoded(e, raw);
     } else {
       prepare_rows(e, raw, ldq);
-      const int* table = e.table(group);
-      const int width = e.width(group);
-      att = e.take((long)N * ldo * e.esize);
-      // the matrix-core kernels take rows that are prepared (whatever prepared them), keys and values of one head
-      // size, and a bias on the scores as a table over the distance (no slopes)
-      const bool matrix_sizes = hd % 16 == 0 && hd <= 128;
-      const bool fast_bf16 = e.bf16_run && !slopes && vd == hd && (!bias || (bias_t && matrix_sizes));
-      if (fast_bf16 && a.max_q > 1 && matrix_sizes) {
-        // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
-        // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
-        // matrix-core kernel
-        const int lead = a.lead_single >= 2 ? a.lead_single : 0;
-        if (lead) decode_attention(e, raw, ldq, lead, a.pos, a.row_req, att);
-        const int rows = N - lead, reqs = a.n_req - lead;
-        const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), nh, a.max_seq, window) : 1;
-        float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(N, nh, hd, n_splits) * 4) : nullptr;
-        RUN(e, gibbs_attention_prefill_bias(raw, kpages, vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
-                                            width, page_size, num_pages, rows, nh, nkv, hd, ldq, ldo, scale, window, n_splits, lead,
-                                            prefill_heads(rows, reqs, nh, nkv, hd, a.max_seq, n_splits), bias_t, bias_len, a.stream));
-        e.give(partial);
-      } else if (fast_bf16 && a.max_q == 1 && hd % 8 == 0) {
-        decode_attention(e, raw, ldq, N, a.pos, a.row_req, att);
-      } else {
-        RUN(e, gibbs_attention_plain_general(raw, kpages, vpages, att, e.p.dtype, a.pos, a.row_req, table, width, page_size, num_pages,
-                                             N, nh, nkv, hd, vd, ldq, ldo, scale, window, slopes, bias, bias_len, a.stream));
-      }
+      att = attend_prepared(e, paged(), raw, ldq, ldo);
     }
     return att;
   }
@@ -717,6 +795,83 @@ struct TimeMixBody : Body {
   }
 };
 
+// ---- latent attention
+// Keys and values of all heads come from one small latent per token: c = rms_norm(W_dkv h)[:rank] and a rotated key part
+// k_r = rotate(W_dkv h)[rank : rank + rot] that all heads share; only [c | k_r] is cached, one row per token.  Head i's key is
+// [W_uk,i c | k_r], its value W_uv,i c, its query [q_i (dim) | rotate(q_r,i) (rot)], with q = W_uq rms_norm(W_dq h) (or W_q h).
+// The scores and the weighted values are taken on the cached rows themselves: q_i . W_uk,i c = (W_uk,i^T q_i) . c, so
+// the queries become [W_uk,i^T q_i | rotate(q_r,i)] (rank + rot entries) and every head attends over the same rows
+// (one kv head of size rank + rot whose values are the rows again); the weighted sum of the latents then goes
+// through W_uv,i.  Softmax over a window, optionally with a sink per head; optionally a sigmoid gate on the heads'
+// outputs from the mixer's input; the out-projection.
+// One product gives [q or W_dq h | W_dkv h | gate] of the normed rows (segments start at multiples of 8 values).
+struct LatentBody : Body {
+  Matrix in, uq, out;                 // uq.w null: queries come straight from `in`
+  const void* uk_t = nullptr;         // [heads][rank][dim]: W_uk of every head, transposed
+  const void* uv = nullptr;           // [heads][vdim][rank]
+  const float* q_gain = nullptr;      // [q_rank]
+  const float* kv_gain = nullptr;     // [rank]
+  const float* sink = nullptr;        // [heads] or null
+  const float* inv_freq = nullptr;    // [rot_dims / 2]
+  int H = 0, D = 0, R = 0, V = 0, C = 0, q_rank = 0, rot_dims = 0, variant = 0, window = 0;
+  int off_kv = 0, off_g = -1;         // where W_dkv h and the gate start in a projected row (off_g < 0: no gate)
+  float scale = 0.f, eps = 0.f;
+  void* pages = nullptr;              // [num_pages, 1, page_size, rank + rot]
+  int num_pages = 0, page_size = 0, group = 0;
+  int cache_group() const override { return group; }
+  Pending general(Exec& e, void* h) const override {
+    const GibbsStepArgs& a = e.a;
+    const int N = a.n_rows, L = C + R;
+    char* raw = (char*)e.linear(h, in, N, false, false, false, nullptr);
+    void* q = raw;
+    long ld_q = in.O;
+    if (uq.w) {
+      void* cq = e.take((long)N * q_rank * e.esize);
+      RUN(e, gibbs_rms_rows_ld(raw, in.O, q_gain, eps, cq, q_rank, e.p.dtype, N, q_rank, a.stream));
+      q = e.linear(cq, uq, N, false, false, false, nullptr);
+      ld_q = uq.O;
+      e.give(cq);
+    }
+    void* q_lat = e.take((long)N * H * L * e.esize);
+    RUN(e, gibbs_latent_prepare(raw + (long)off_kv * e.esize, in.O, q, ld_q, q_lat, (long)H * L, pages, e.p.dtype, kv_gain, eps, inv_freq,
+                                rot_dims, variant, a.pos, a.row_req, e.table(group), e.width(group), page_size, num_pages, N, H, D, R, C,
+                                a.stream));
+    RUN(e, gibbs_gemm_heads(q, ld_q, D + R, uk_t, (long)C * D, D, q_lat, (long)H * L, L, e.p.dtype, N, C, D, H, a.stream));
+    if (uq.w) e.give(q);
+    const PagedAttention t{pages, pages, num_pages, page_size, group, H, 1, L, L, scale, window, nullptr, nullptr, nullptr, 0, sink};
+    void* att = attend_prepared(e, t, q_lat, (long)H * L, (long)H * L);
+    e.give(q_lat);
+    void* o = e.take((long)N * H * V * e.esize);
+    RUN(e, gibbs_gemm_heads(att, (long)H * L, L, uv, (long)V * C, C, o, (long)H * V, V, e.p.dtype, N, V, C, H, a.stream));
+    e.give(att);
+    if (off_g >= 0) RUN(e, gibbs_sigmoid_gate(o, (long)H * V, raw + (long)off_g * e.esize, in.O, e.p.dtype, N, H * V, a.stream));
+    e.give(raw);
+    Pending delta;
+    delta.data = e.linear(o, out, N, false, true, true, &delta.parts);
+    e.give(o);
+    return delta;
+  }
+};
+
+// ---- dense feed-forward without a gate: down(act(up h)), act a polynomial of row-normed powers
+struct MlpBody : Body {
+  Matrix up, down;
+  int F = 0;
+  const float* coef = nullptr;        // [4] on the device: a, b, c, e of a N(z) + b N(z^2) + c N(z^3) + e
+  float eps = 0.f;
+  Pending general(Exec& e, void* h) const override {
+    const int N = e.a.n_rows;
+    void* z = e.linear(h, up, N, false, false, false, nullptr);
+    void* y = e.take((long)N * F * e.esize);
+    RUN(e, gibbs_poly_norm(z, y, e.p.dtype, coef, eps, N, F, e.a.stream));
+    e.give(z);
+    Pending delta;
+    delta.data = e.linear(y, down, N, false, true, true, &delta.parts);
+    e.give(y);
+    return delta;
+  }
+};
+
 // ---- a body from elsewhere
 struct HostBody : Body {
   GibbsHostBody fn = nullptr;
@@ -738,7 +893,16 @@ void Exec::run() {
   float* x = a.x_in;
   void* mirror = few_rows ? a.mirror_in : nullptr;
   float* embedded = nullptr;     // the embedding's output, for a program that adds it again
-  if (!x) {
+  const int S = p.streams;
+  if (!x && p.table_sums()) {
+    // the token table's row plus the pair table's and the position table's, into every stream; then the requests' last
+    // tokens go to their slots, for the first row of their next portion
+    x = (float*)take((long)S * N * H * 4);
+    mirror = nullptr;
+    RUN(*this, gibbs_embed_tables(p.table, p.pair_table, p.pos_table, p.table_dtype, a.ids, a.pos, a.row_req, a.cu, a.slot, p.prev_state,
+                                  p.prev_stride, x, S, N, H, p.vocab, p.buckets, p.mul_prev, p.mul_cur, p.pos_len, a.stream));
+    if (p.pair_table) RUN(*this, gibbs_store_last_token(a.ids, a.cu, a.slot, p.prev_state, p.prev_stride, a.n_req, a.stream));
+  } else if (!x) {
     x = (float*)take((long)N * H * 4);
     mirror = few_rows ? take((long)N * H * 2) : nullptr;
     if (p.reinjects) embedded = (float*)take((long)N * H * 4);
@@ -806,6 +970,18 @@ void Exec::run() {
         give(mirror);
         mirror = nullptr;
         break;
+      case Plan::OP_STREAMS_NORM:
+        rows[op.result] = p.norms[op.norm]->run_streams(*this, x, S, p.hypers[op.body].in, nullptr, N);
+        break;
+      case Plan::OP_STREAMS_ADD: {
+        const Hyper& hc = p.hypers[op.body];
+        Pending& d = deltas[op.value];
+        RUN(*this, gibbs_streams_write(x, S, (long)N * H, hc.mix, hc.out, d.data, d.parts >= 2 ? GIBBS_F32 : p.dtype, std::max(d.parts, 1),
+                                       (long)N * H, (long)N * H, a.stream));
+        give(d.data);
+        d = Pending{};
+        break;
+      }
       case Plan::OP_DROP:
         give(rows[op.value]);
         give(deltas[op.value].data);
@@ -815,7 +991,9 @@ void Exec::run() {
     }
   }
   if (whole && a.n_logits > 0 && ok()) {
-    void* h = p.norms[p.tail]->run(*this, x, pending, a.logit_rows, a.n_logits);
+    // (several streams: the model's output is their sum)
+    void* h = S > 1 ? p.norms[p.tail]->run_streams(*this, x, S, nullptr, a.logit_rows, a.n_logits)
+                    : p.norms[p.tail]->run(*this, x, pending, a.logit_rows, a.n_logits);
     linear_into(h, p.head, a.n_logits, true, true, a.logits);   // the head: float32 logits straight into the caller's buffer
     give(h);
   }
@@ -842,9 +1020,17 @@ int check_args(const Plan* p, const GibbsStepArgs* a, bool whole_step) {
     GIBBS_REQUIRE(p->has_norm(p->tail) && p->head.w, "step: logits are wanted and the plan has no final norm or no head");
     GIBBS_REQUIRE(a->workspace == nullptr || a->logits, "step: logits are wanted and there is no buffer for them");
   }
+  GIBBS_REQUIRE(!p->table_sums() || (p->embed_scale == 1.0f && !p->embed_inv_freq && !p->reinjects), "step: an embedding with a pair or position table, or several streams, takes no scale, sinusoid or second addition");
+  GIBBS_REQUIRE(!a->x_in || !p->table_sums() || a->n_ops, "step: this model's embedding is more than the token table's rows: the step embeds its rows itself");
+  GIBBS_REQUIRE(!p->pair_table || (p->prev_state && a->slot && a->cu && a->row_req), "step: the pair table needs the requests' slots");
   const int first = a->n_ops ? a->first_op : 0, last = a->n_ops ? a->first_op + a->n_ops : (int)p->ops.size();
   for (int i = first; i < last; ++i) {
     const Plan::Op& op = p->ops[i];
+    const bool of_streams = op.kind == Plan::OP_STREAMS_NORM || op.kind == Plan::OP_STREAMS_ADD;
+    const bool of_one = op.kind == Plan::OP_HALF || op.kind == Plan::OP_NORM || op.kind == Plan::OP_ADD || op.kind == Plan::OP_ADD_NORMED ||
+                        op.kind == Plan::OP_REINJECT;
+    GIBBS_REQUIRE(p->streams == 1 || !of_one, "step: operation %d works on one residual stream, the plan has %d", i, p->streams);
+    GIBBS_REQUIRE(!of_streams || p->streams <= 8, "step: %d residual streams (1 to 8)", p->streams);
     if (op.kind != Plan::OP_HALF && op.kind != Plan::OP_BODY) continue;
     const int g = p->bodies[op.body]->cache_group();
     GIBBS_REQUIRE(g < 0 || (g < a->n_groups && a->tables && a->tables[g] && a->widths[g] > 0), "step: no block table for cache group %d", g);
@@ -955,6 +1141,77 @@ GIBBS_EXPORT int gibbs_plan_body_host(void* plan, GibbsHostBody fn, void* user, 
   b->fn = fn; b->user = user; b->group = group;
   p->bodies.push_back(std::move(b));
   return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_norm_layer(void* plan, const float* gain, const float* bias, float eps) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  auto n = std::make_unique<LayerNorm>();
+  n->gain = gain; n->bias = bias; n->eps = eps;
+  p->norms.push_back(std::move(n));
+  return (int)p->norms.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_latent(void* plan, const GibbsLatentSpec* d) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!d || !(d->w_in && d->w_out && d->w_uk_t && d->w_uv && d->pages && d->heads > 0 && d->dim > 0 && d->rot >= 0 && d->vdim > 0 &&
+              d->rank > 0 && d->in_rows > 0 && d->off_kv >= 0 && d->off_kv + d->rank + d->rot <= d->in_rows && d->num_pages > 0 &&
+              d->page_size > 0 && d->group >= 0 && d->window >= 0 && (d->rot_dims == 0 || d->inv_freq) && d->rot_dims <= d->rot &&
+              (!d->w_uq || d->q_rank > 0) && (d->off_g < 0 || d->off_g + d->heads * d->vdim <= d->in_rows))) {
+    gibbs_fail("plan: bad latent attention");
+    return -1;
+  }
+  if (d->rank + d->rot > 512) { gibbs_fail("plan: a cached row of %d values (latent + rotated key part) is more than the attention kernels take (512)", d->rank + d->rot); return -1; }
+  auto b = std::make_unique<LatentBody>();
+  b->in = Matrix{d->w_in, nullptr, d->in_rows, p->hidden};
+  if (d->w_uq) b->uq = Matrix{d->w_uq, nullptr, d->heads * (d->dim + d->rot), d->q_rank};
+  b->out = Matrix{d->w_out, nullptr, p->hidden, d->heads * d->vdim};
+  b->uk_t = d->w_uk_t; b->uv = d->w_uv; b->q_gain = d->q_gain; b->kv_gain = d->kv_gain; b->sink = d->sink; b->inv_freq = d->inv_freq;
+  b->H = d->heads; b->D = d->dim; b->R = d->rot; b->V = d->vdim; b->C = d->rank; b->q_rank = d->q_rank; b->rot_dims = d->rot_dims;
+  b->variant = d->variant; b->window = d->window; b->off_kv = d->off_kv; b->off_g = d->off_g; b->scale = d->scale; b->eps = d->eps;
+  b->pages = d->pages; b->num_pages = d->num_pages; b->page_size = d->page_size; b->group = d->group;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_mlp(void* plan, const void* w_up, const void* w_down, int F, const float* coef, float eps) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!(w_up && w_down && coef && F > 0)) { gibbs_fail("plan: bad feed-forward width %d", F); return -1; }
+  auto b = std::make_unique<MlpBody>();
+  b->up = Matrix{w_up, nullptr, F, p->hidden};
+  b->down = Matrix{w_down, nullptr, p->hidden, F};
+  b->F = F; b->coef = coef; b->eps = eps;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_streams(void* plan, int streams) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (streams < 1 || streams > 8) { gibbs_fail("plan: %d residual streams (1 to 8)", streams); return -1; }
+  p->streams = streams;
+  return 0;
+}
+GIBBS_EXPORT int gibbs_plan_hyper(void* plan, const float* in, const float* mix, const float* out) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!(in && mix && out)) { gibbs_fail("plan: a hyper-connection needs its three tensors"); return -1; }
+  p->hypers.push_back(Hyper{in, mix, out});
+  return (int)p->hypers.size() - 1;
+}
+GIBBS_EXPORT int gibbs_plan_embedding_tables(void* plan, const void* pair_table, int buckets, int mul_prev, int mul_cur,
+                                             const void* pos_table, int pos_len, int* prev_state, long prev_stride) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if ((pair_table && (buckets <= 0 || !prev_state || prev_stride <= 0)) || (pos_table && pos_len <= 0)) {
+    gibbs_fail("plan: bad embedding tables (buckets %d, positions %d)", buckets, pos_len);
+    return -1;
+  }
+  p->pair_table = pair_table; p->buckets = buckets; p->mul_prev = mul_prev; p->mul_cur = mul_cur;
+  p->pos_table = pos_table; p->pos_len = pos_len; p->prev_state = prev_state; p->prev_stride = prev_stride;
+  return 0;
 }
 
 // ---- more about parts that are there already
@@ -1092,6 +1349,18 @@ GIBBS_EXPORT int gibbs_plan_op_add_normed(void* plan, int norm, int value) {
   if (!p) return -1;
   if (!p->has_norm(norm) || !known_value(p, value)) { gibbs_fail("plan: norm %d of value %d: no such part or value", norm, value); return -1; }
   return append(p, Plan::OP_ADD_NORMED, norm, -1, value, false);
+}
+GIBBS_EXPORT int gibbs_plan_op_streams_norm(void* plan, int norm, int hyper) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!p->has_norm(norm) || !p->has_hyper(hyper)) { gibbs_fail("plan: norm %d of hyper-connection %d: no such part", norm, hyper); return -1; }
+  return append(p, Plan::OP_STREAMS_NORM, norm, hyper, -1, true);
+}
+GIBBS_EXPORT int gibbs_plan_op_streams_add(void* plan, int hyper, int value) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!p->has_hyper(hyper) || !known_value(p, value)) { gibbs_fail("plan: hyper-connection %d of value %d: no such part or value", hyper, value); return -1; }
+  return append(p, Plan::OP_STREAMS_ADD, -1, hyper, value, false);
 }
 GIBBS_EXPORT int gibbs_plan_op_reinject(void* plan) {
   Plan* p = open_plan(plan);

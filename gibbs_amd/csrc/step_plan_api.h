@@ -110,6 +110,40 @@ struct GibbsTimeMixSpec {
 };
 int gibbs_plan_body_time_mix(void* plan, const struct GibbsTimeMixSpec* spec);
 
+// Layer norm with gain and bias (either may be null: 1 and 0).
+int gibbs_plan_norm_layer(void* plan, const float* gain, const float* bias, float eps);
+
+// Latent attention: one cached row [latent (rank) | rotated key part (rot)] per token, shared by all heads.  w_in
+// [in_rows, hidden]: the rows of the queries (heads * (dim + rot); or, with w_uq [heads * (dim + rot), q_rank], the q_rank
+// rows of the queries' own latent, which is RMS-normed with q_gain), at off_kv the rank + rot rows of the keys' and values'
+// down-projection (the first rank RMS-normed with kv_gain), at off_g (< 0: none) the heads * vdim rows of a sigmoid gate on
+// the heads' outputs.  w_uk_t [heads, rank, dim]: every head's key up-projection, transposed; w_uv [heads * vdim, rank].
+// A query head is [dim unrotated | rot rotated]; the first rot_dims entries of a rotated part turn with the position
+// (variant 0: pairs (i, i + rot_dims / 2), 1: pairs (2 i, 2 i + 1); inv_freq [rot_dims / 2]).  window 0: all keys;
+// sink [heads] or null: a term exp(sink[h]) in the softmax's denominator.  pages: [num_pages, page_size, rank + rot].
+struct GibbsLatentSpec {
+  const void* w_in; const void* w_uq; const void* w_uk_t; const void* w_uv; const void* w_out;
+  const float* q_gain; const float* kv_gain; const float* sink; const float* inv_freq;
+  void* pages;
+  int in_rows, heads, dim, rot, vdim, rank, q_rank, rot_dims, variant, window, off_kv, off_g, num_pages, page_size, group;
+  float scale, eps;
+};
+int gibbs_plan_body_latent(void* plan, const struct GibbsLatentSpec* spec);
+// Dense feed-forward without a gate: down(act(up h)), act(z) = a N(z) + b N(z^2) + c N(z^3) + e with coef = [a, b, c, e]
+// on the device and N the division of a row by its root mean square (eps inside the root).
+int gibbs_plan_body_mlp(void* plan, const void* w_up, const void* w_down, int F, const float* coef, float eps);
+
+// Several residual streams (1 to 8): every stream starts as the embedding's output, sublayers read and write them
+// through hyper-connections (in [streams], mix [streams, streams] indexed [from][to], out [streams]), and the model's
+// output is the streams' sum.
+int gibbs_plan_streams(void* plan, int streams);
+int gibbs_plan_hyper(void* plan, const float* in, const float* mix, const float* out);
+// Rows of further tables added to the token table's: pair_table [buckets + 1, hidden], row (previous token * mul_prev +
+// token * mul_cur) mod buckets, row `buckets` for a sequence's first token (the previous token of a request's earlier step
+// lives at prev_state[slot * prev_stride]); pos_table [pos_len, hidden], row = position.  Either may be null.
+int gibbs_plan_embedding_tables(void* plan, const void* pair_table, int buckets, int mul_prev, int mul_cur,
+                                const void* pos_table, int pos_len, int* prev_state, long prev_stride);
+
 // ---- the program (values are normed rows or deltas, named by the index their operation returns)
 int gibbs_plan_op_half(void* plan, int norm, int body);       // x += body(norm(x)), in fused kernels where it can
 int gibbs_plan_op_norm(void* plan, int norm);                 // -> value: norm(x + what is pending)
@@ -118,6 +152,8 @@ int gibbs_plan_op_add(void* plan, int value);                 // x += delta (laz
 int gibbs_plan_op_drop(void* plan, int value);                // the value is not read again
 int gibbs_plan_op_norm_delta(void* plan, int norm, int value);   // -> value: norm(a body's delta), the stream untouched
 int gibbs_plan_op_add_normed(void* plan, int norm, int value);   // x += norm(a body's delta), in one pass where the norm can
+int gibbs_plan_op_streams_norm(void* plan, int norm, int hyper);   // -> value: norm(sum_s in[s] x_s)
+int gibbs_plan_op_streams_add(void* plan, int hyper, int value);   // x_t <- sum_s mix[s][t] x_s + out[t] delta, all t at once
 int gibbs_plan_op_reinject(void* plan);                       // x += the embedding's output (what the step's first operation saw)
 int gibbs_plan_tail(void* plan, int norm);                    // the norm in front of the head
 int gibbs_plan_op_count(const void* plan);

@@ -89,7 +89,9 @@ class Engine:
         for owner, ((run, role), src) in enumerate(zip(self.model.cache_owners(), self.model.kv_sources())):
             self._views[run][role] = self.device_cache.layer_view(owner, src)
         self._stager = BatchStager(self.device)
-        self.plan = NativePlan.build(self.model, self._views, self.rt)
+        own = self.model.model_state_owner()
+        self.plan = NativePlan.build(self.model, self._views, self.rt,
+                                     model_view=None if own is None else self.device_cache.layer_view(own))
 
     # ------------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> bool:

@@ -1,8 +1,8 @@
 """Parts that layers are put together from; importing this package registers the built-in kinds."""
-from .base import (ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, Block, FeedForward, Mixer, Norm, Part,
+from .base import (ARRANGEMENTS, CONNECTIONS, Connection, register_connection, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, Block, FeedForward, Mixer, Norm, Part,
                    PositionEncoding, Rotation, Runtime, build_block, build_feed_forward, build_mixer, build_norm,
                    build_position, register_arrangement, register_feed_forward, register_mixer, register_norm,
                    register_position)
-from . import attention, block, delta, distance_bias, glu, norm, rope, shortconv, timemix  # noqa: F401  (registration)
+from . import attention, block, delta, distance_bias, glu, latent, mlp, norm, rope, shortconv, timemix  # noqa: F401  (registration)
 from .model import DecoderModel
 from .native import NativePlan

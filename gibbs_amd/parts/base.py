@@ -13,6 +13,7 @@ kind in a spec; nothing else in the framework changes.
                   that are added in order); may ask for cache pages (`cache_need`) and
                   per-request state of fixed size (`state_needs`)
   FeedForward     forward(h, batch) -> delta [N, hidden]
+  Connection      how a sublayer reads and writes several residual streams
   Block           emit(plan, caches): the arrangement of a layer's parts, as operations of the plan
 
 A part written with tensor operations implements `forward` and nothing else: the base class's
@@ -31,7 +32,7 @@ from typing import Callable, Dict, List, Mapping, Optional, Sequence, Type
 import torch
 
 from ..cache.needs import CacheNeed, StateNeed
-from ..config.spec import FeedForwardSpec, LayerSpec, MixerSpec, NormSpec, PositionSpec
+from ..config.spec import ConnectionSpec, FeedForwardSpec, LayerSpec, MixerSpec, NormSpec, PositionSpec
 from ..weights.loader import TensorDecl, WeightStore
 
 
@@ -213,8 +214,21 @@ class FeedForward(Part):
         return solo[0].body_forward(solo[1], h.contiguous(), batch)
 
 
+class Connection(Part):
+    """How a sublayer reads and writes the model's residual streams (`ConnectionSpec`)."""
+
+    def __init__(self, spec: ConnectionSpec):
+        self.spec, self.streams = spec, int(spec.streams)
+
+    def emit(self, plan) -> int:
+        """Lays the connection down in `plan`; returns its number there."""
+        raise NotImplementedError
+
+
 def build_part(spec, hidden: int, layer_index: int) -> Part:
     """The part that a spec of any of the layer's kinds describes."""
+    if isinstance(spec, ConnectionSpec):
+        return _lookup(CONNECTIONS, spec.kind, "connection")(spec)
     if isinstance(spec, NormSpec):
         return build_norm(spec, hidden)
     if isinstance(spec, MixerSpec):
@@ -293,6 +307,7 @@ POSITIONS: Dict[str, Type[PositionEncoding]] = {}
 MIXERS: Dict[str, Type[Mixer]] = {}
 FEED_FORWARDS: Dict[str, Type[FeedForward]] = {}
 ARRANGEMENTS: Dict[str, Type[Block]] = {}
+CONNECTIONS: Dict[str, Type[Connection]] = {}
 
 
 def _register(table: Dict[str, type], kind: str) -> Callable[[type], type]:
@@ -307,6 +322,7 @@ def register_position(kind: str): return _register(POSITIONS, kind)
 def register_mixer(kind: str): return _register(MIXERS, kind)
 def register_feed_forward(kind: str): return _register(FEED_FORWARDS, kind)
 def register_arrangement(kind: str): return _register(ARRANGEMENTS, kind)
+def register_connection(kind: str): return _register(CONNECTIONS, kind)
 
 
 def _lookup(table: Dict[str, type], kind: str, what: str) -> type:

@@ -17,7 +17,8 @@ from __future__ import annotations
 
 import torch
 
-from .base import Block, Runtime, register_arrangement
+from ..weights.loader import FLOAT32, TensorDecl
+from .base import Block, Connection, Runtime, register_arrangement, register_connection
 
 
 @register_arrangement("pre_norm")
@@ -98,3 +99,61 @@ class ParallelNormsBlock(Block):
             delta = plan.apply(self.mixer.emit(plan, caches["mixer"]), h)
             plan.drop(h)
             plan.add(delta)
+
+
+@register_connection("hyper")
+class HyperConnection(Connection):
+    """A sublayer over S residual streams x_1 .. x_S: it reads u = sum_s in[s] x_s and, with its result y, writes all
+    streams at once from the old ones, x_t <- sum_s mix[s, t] x_s + out[t] y (`mix` indexed [from, to]).  The three
+    tensors are float32; the streams and both sums are float32 in either precision of a run."""
+
+    def tensor_decls(self):
+        t, S = self.spec.tensors, self.streams
+        return [TensorDecl(t["in"], (S,), FLOAT32, init="gain"), TensorDecl(t["out"], (S,), FLOAT32, init="gain"),
+                TensorDecl(t["mix"], (S, S), FLOAT32)]
+
+    def bind(self, weights, rt: Runtime) -> None:
+        self.rt = rt
+        t = self.spec.tensors
+        self.w_in, self.w_mix, self.w_out = weights[t["in"]], weights[t["mix"]].contiguous(), weights[t["out"]]
+
+    def small_tensors(self):
+        return [self.w_in, self.w_mix, self.w_out]
+
+    def emit(self, plan) -> int:
+        return plan.hyper(self.w_in, self.w_mix, self.w_out)
+
+
+@register_arrangement("sublayers")
+class SublayersBlock(Block):
+    """Pre-norm sublayers, each of which may be missing but the first: x += mixer(norm1(x)); x += ffn(norm2(x)).
+
+    Roles: `norm1`, `mixer`, and optionally `norm2` with `ffn`.  With `connection1` (and `connection2` for the
+    feed-forward) the model has several residual streams, and a sublayer reads and writes them through its
+    connection instead of adding into one: y = sublayer(norm(read(streams))); write(streams, y)."""
+
+    def __init__(self, spec, hidden, layer_index):
+        super().__init__(spec, hidden, layer_index)
+        self.has_ffn = "ffn" in self.named
+        self.connected = "connection1" in self.named
+        want = ["norm1", "mixer"] + (["norm2"] if self.has_ffn else []) + (["connection2"] if self.has_ffn and self.connected else [])
+        missing = [r for r in want if r not in self.named]
+        if missing:
+            raise ValueError(f"layer {spec.name!r} lacks the parts {missing}")
+
+    def streams(self) -> int:
+        return self.connection1.streams if self.connected else 1
+
+    def emit(self, plan, caches) -> None:
+        subs = [(self.norm1, lambda: self.mixer.emit(plan, caches["mixer"]), "connection1")]
+        if self.has_ffn:
+            subs.append((self.norm2, lambda: self.ffn.emit(plan), "connection2"))
+        for norm, body, role in subs:
+            if self.connected:
+                c = self.named[role].emit(plan)
+                h = plan.streams_normed(norm.emit(plan), c)
+                delta = plan.apply(body(), h)
+                plan.drop(h)
+                plan.streams_add(c, delta)
+            else:
+                plan.half(norm.emit(plan), body())

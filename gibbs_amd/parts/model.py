@@ -15,11 +15,13 @@ import torch
 from .. import ops
 from ..cache.needs import CacheNeed, StateNeed
 from ..config.spec import ModelSpec
-from ..weights.loader import TensorDecl, WeightStore
+from ..weights.loader import FLOAT32, TensorDecl, WeightStore
 from .base import Block, Part, Runtime, build_block, build_norm
 
 
 class DecoderModel(Part):
+    PREV_TOKEN = "previous_token"      # state the model itself keeps per request: its last token (for a table over token pairs)
+
     def __init__(self, spec: ModelSpec):
         self.spec = spec
         self.blocks: List[Block] = [build_block(ls, spec.hidden, i) for i, ls in enumerate(spec.layers)]
@@ -53,7 +55,20 @@ class DecoderModel(Part):
             decls += b.tensor_decls()
         if s.head is not None:
             decls.append(TensorDecl(s.head, (s.vocab, s.hidden)))
+        tables = s.embedding_tables
+        if tables is not None and tables.pair is not None:
+            decls.append(TensorDecl(tables.pair, (tables.buckets + 1, s.hidden)))
+        if tables is not None and tables.position is not None:
+            decls.append(TensorDecl(tables.position, (tables.positions, s.hidden)))
+        decls += [TensorDecl(name, tuple(shape), FLOAT32 if len(shape) <= 2 else "compute") for name, shape in s.unread_tensors]
         return decls
+
+    def model_state_needs(self) -> Sequence[StateNeed]:
+        """Per-request state of fixed size that the model itself keeps, beside its mixers'."""
+        tables = self.spec.embedding_tables
+        if tables is not None and tables.pair is not None:
+            return (StateNeed(self.PREV_TOKEN, (), "int32"),)
+        return ()
 
     # Caches belong to the mixers of runs (entries of the run order), not to layers: a layer that the
     # order names twice shares its weights between both runs, but each run caches its own keys,
@@ -65,11 +80,18 @@ class DecoderModel(Part):
     def _mixer(self, owner: Tuple[int, str]):
         return self.blocks[self.spec.order[owner[0]]].mixers()[owner[1]]
 
+    # What the cache manager is asked for: one entry per cache owner and, when the model itself keeps state per
+    # request, one more entry behind them (no pages, the model's states): entry `model_state_owner()`.
     def cache_needs(self) -> List[Optional[CacheNeed]]:
-        return [self._mixer(o).cache_need() for o in self.cache_owners()]
+        own = [None] if self.model_state_needs() else []
+        return [self._mixer(o).cache_need() for o in self.cache_owners()] + own
 
     def state_needs(self) -> List[Sequence[StateNeed]]:
-        return [tuple(self._mixer(o).state_needs()) for o in self.cache_owners()]
+        own = [tuple(self.model_state_needs())] if self.model_state_needs() else []
+        return [tuple(self._mixer(o).state_needs()) for o in self.cache_owners()] + own
+
+    def model_state_owner(self) -> Optional[int]:
+        return len(self.cache_owners()) if self.model_state_needs() else None
 
     def kv_sources(self) -> List[Optional[int]]:
         """For each cache owner, the earlier owner whose pages it reads (the page-owning mixer of the
@@ -99,6 +121,12 @@ class DecoderModel(Part):
             width = self.spec.hidden
             i = torch.arange(width // 2, dtype=torch.float64)
             self.embedding_inv_freq = (float(pos.params.get("base", 10000.0)) ** (-2.0 * i / width)).to(torch.float32).to(rt.device)
+        tables = self.spec.embedding_tables
+        self.pair_table = weights[tables.pair] if tables is not None and tables.pair is not None else None
+        self.position_table = weights[tables.position] if tables is not None and tables.position is not None else None
+        streams = {b.streams() for b in self.blocks if hasattr(b, "streams")}
+        if streams - {self.spec.streams} or (self.spec.streams != 1 and len(streams) != 1):
+            raise ValueError(f"the model has {self.spec.streams} residual streams, its layers are connected for {sorted(streams)}")
         self.final_norm.bind(weights, rt)
         for b in self.blocks:
             b.bind(weights, rt)

@@ -52,6 +52,15 @@ class TimeMixSpec(ctypes.Structure):
                 ("heads", c_int), ("dim", c_int), ("rank", c_int), ("eps", ctypes.c_float)]
 
 
+class LatentSpec(ctypes.Structure):
+    """GibbsLatentSpec of csrc/step_plan_api.h."""
+    _fields_ = [("w_in", c_void_p), ("w_uq", c_void_p), ("w_uk_t", c_void_p), ("w_uv", c_void_p), ("w_out", c_void_p),
+                ("q_gain", c_void_p), ("kv_gain", c_void_p), ("sink", c_void_p), ("inv_freq", c_void_p), ("pages", c_void_p),
+                ("in_rows", c_int), ("heads", c_int), ("dim", c_int), ("rot", c_int), ("vdim", c_int), ("rank", c_int),
+                ("q_rank", c_int), ("rot_dims", c_int), ("variant", c_int), ("window", c_int), ("off_kv", c_int), ("off_g", c_int),
+                ("num_pages", c_int), ("page_size", c_int), ("group", c_int), ("scale", ctypes.c_float), ("eps", ctypes.c_float)]
+
+
 HOST_BODY = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p)
 HOST_NORM = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p)
 HOST_ROWS = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_long)
@@ -79,6 +88,14 @@ def declare(lib) -> None:
         "gibbs_plan_glu_clamped": ([P, I, F, F], I),
         "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
         "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
+        "gibbs_plan_norm_layer": ([P, P, P, F], I),
+        "gibbs_plan_body_latent": ([P, POINTER(LatentSpec)], I),
+        "gibbs_plan_body_mlp": ([P, P, P, I, P, F], I),
+        "gibbs_plan_streams": ([P, I], I),
+        "gibbs_plan_hyper": ([P, P, P, P], I),
+        "gibbs_plan_embedding_tables": ([P, P, I, I, I, P, I, P, LG], I),
+        "gibbs_plan_op_streams_norm": ([P, I, I], I),
+        "gibbs_plan_op_streams_add": ([P, I, I], I),
         "gibbs_plan_op_norm_delta": ([P, I, I], I),
         "gibbs_plan_op_add_normed": ([P, I, I], I),
         "gibbs_plan_op_reinject": ([P], I),
@@ -155,6 +172,10 @@ class NativePlan:
     def rms_norm(self, gain: Optional[torch.Tensor], eps: float) -> int:
         (g,) = self._held(gain)
         return self._made(L.library().gibbs_plan_norm_rms(self.handle, g, float(eps)))
+
+    def layer_norm(self, gain: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float) -> int:
+        g, b = self._held(gain, bias)
+        return self._made(L.library().gibbs_plan_norm_layer(self.handle, g, b, float(eps)))
 
     def host_norm(self, forward: Callable) -> int:
         """A norm written with tensor operations: `forward(x, delta, rows, n_rows) -> normed rows` (the
@@ -273,6 +294,64 @@ class NativePlan:
         d.heads, d.dim, d.rank, d.eps = m.heads, m.dim, m.rank, m.norm_eps
         return self._made(L.library().gibbs_plan_body_time_mix(self.handle, ctypes.byref(d)))
 
+    def latent_attention(self, m, *, pages: torch.Tensor, group: int) -> int:
+        """The latent-attention mixer `m` (parts/latent.py) over its pages [num_pages, 1, page_size, kv_rank + rot_dim]."""
+        from ..ops import ROPE_VARIANTS
+        assert pages.is_contiguous() and pages.dtype == self.rt.act_dtype
+        d = LatentSpec()
+        d.w_in, d.w_uq, d.w_uk_t, d.w_uv, d.w_out = self._held(m.w_in, m.w_uq, m.w_uk_t, m.w_uv, m.w_out)
+        d.q_gain, d.kv_gain, d.sink = self._held(m.q_gain, m.kv_gain, m.sinks)
+        d.rot_dims = d.variant = 0
+        if m.rot is not None:
+            (d.inv_freq,) = self._held(m.rot.inv_freq)
+            d.rot_dims, d.variant = int(m.rot.rotary_dim), ROPE_VARIANTS[m.rot.variant]
+        d.pages = pages.data_ptr()
+        self.keep.append(pages)
+        d.in_rows, d.heads, d.dim, d.rot, d.vdim, d.rank, d.q_rank = m.w_in.shape[0], m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank, m.q_rank
+        d.window, d.off_kv, d.off_g = int(m.window or 0), m.off_kv, m.off_g
+        d.num_pages, d.page_size, d.group = int(pages.shape[0]), int(pages.shape[2]), int(group)
+        d.scale, d.eps = m.scale, m.norm_eps
+        return self._made(L.library().gibbs_plan_body_latent(self.handle, ctypes.byref(d)))
+
+    def mlp(self, *, w_up, w_down, inter: int, coef: torch.Tensor, eps: float) -> int:
+        """down(act(up h)) with the polynomial-norm activation; coef: float32 [4] on the device."""
+        assert coef.dtype == torch.float32 and coef.numel() == 4
+        u, dn, c = self._held(w_up, w_down, coef)
+        return self._made(L.library().gibbs_plan_body_mlp(self.handle, u, dn, int(inter), c, float(eps)))
+
+    def streams(self, n: int) -> None:
+        """The model keeps `n` residual streams, each starting as the embedding's output; its output is their sum."""
+        self._made(L.library().gibbs_plan_streams(self.handle, int(n)))
+        if n > 1:
+            self.plain_embedding = False
+
+    def hyper(self, w_in: torch.Tensor, w_mix: torch.Tensor, w_out: torch.Tensor) -> int:
+        """A hyper-connection: in [streams], mix [streams, streams] indexed [from, to], out [streams], float32."""
+        assert all(t.dtype == torch.float32 and t.is_contiguous() for t in (w_in, w_mix, w_out))
+        return self._made(L.library().gibbs_plan_hyper(self.handle, *self._held(w_in, w_mix, w_out)))
+
+    def embedding_tables(self, *, pair, buckets: int, mul_prev: int, mul_cur: int, position, prev_state) -> None:
+        """Rows of a table over hashed token pairs and of a table over positions, added to the token table's row.
+        `prev_state`: int32 [slots] (a column of the state arena): every request's last token."""
+        pt, ps = self._held(pair, position)
+        stride = 0
+        if pair is not None:
+            assert prev_state is not None and prev_state.dtype == torch.int32 and prev_state.dim() == 1
+            stride = int(prev_state.stride(0))
+            self.keep.append(prev_state)
+        self._made(L.library().gibbs_plan_embedding_tables(
+            self.handle, pt, int(buckets), int(mul_prev), int(mul_cur), ps, 0 if position is None else int(position.shape[0]),
+            None if pair is None else prev_state.data_ptr(), stride))
+        self.plain_embedding = False
+
+    def streams_normed(self, norm: int, hyper: int) -> int:
+        """-> value: norm(sum_s in[s] x_s)."""
+        return self._made(L.library().gibbs_plan_op_streams_norm(self.handle, norm, hyper))
+
+    def streams_add(self, hyper: int, value: int) -> None:
+        """x_t <- sum_s mix[s, t] x_s + out[t] delta for all streams at once; the delta is used up."""
+        self._made(L.library().gibbs_plan_op_streams_add(self.handle, hyper, value))
+
     def host_body(self, forward: Callable, group: Optional[int] = None) -> int:
         """A mixer or feed-forward written with tensor operations: `forward(h, batch) -> delta [N, hidden]`
         (or float32 partial sums [S, N, hidden]).  `group`: the cache group whose block table it reads."""
@@ -331,11 +410,23 @@ class NativePlan:
         return int(L.library().gibbs_plan_op_count(self.handle))
 
     @classmethod
-    def build(cls, model, views, rt) -> "NativePlan":
-        """The plan of a bound `DecoderModel` (`views[run]`: the cache views of the run's mixers by role)."""
+    def build(cls, model, views, rt, model_view=None) -> "NativePlan":
+        """The plan of a bound `DecoderModel` (`views[run]`: the cache views of the run's mixers by role; `model_view`:
+        the view of the state that the model itself keeps per request)."""
         plan = cls(rt, model.spec.hidden, model.spec.vocab, model.table, model.head, model.head_packed)
         if model.spec.embedding_scale != 1.0 or model.embedding_inv_freq is not None:
             plan.embedding(model.spec.embedding_scale, model.embedding_inv_freq)
+        if model.spec.streams != 1:
+            plan.streams(model.spec.streams)
+        tables = model.spec.embedding_tables
+        if tables is not None and (tables.pair is not None or tables.position is not None):
+            prev = None
+            if tables.pair is not None:
+                if model_view is None or model.PREV_TOKEN not in model_view.states:
+                    raise ValueError("a table over token pairs needs the requests' last tokens: no state view was given")
+                prev = model_view.states[model.PREV_TOKEN]
+            plan.embedding_tables(pair=model.pair_table, buckets=tables.buckets, mul_prev=tables.mul_prev, mul_cur=tables.mul_cur,
+                                  position=model.position_table, prev_state=prev)
         for run, i in enumerate(model.spec.order):
             if run in model.spec.reinject_before:
                 plan.reinject()

@@ -1,4 +1,9 @@
-"""RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * gain, eps inside the root, the gain multiplied
+"""Norms over the model's width.
+
+LayerNorm (`"layer"`): out = (x - mean) / sqrt(mean((x - mean)^2) + eps) * gain + bias, all in float32; it also
+norms a weighted sum of several residual streams (what a hyper-connected sublayer reads).
+
+RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * gain, eps inside the root, the gain multiplied
 last, no (1 + gain) offset (src/model/simd.rs:75-110,
 arch/lib/transformer.json5:9-11)."""
 from __future__ import annotations
@@ -31,3 +36,23 @@ class RMSNorm(Norm):
 
     def emit(self, plan) -> int:
         return plan.rms_norm(self.gain, self.spec.eps)
+
+
+@register_norm("layer")
+class LayerNorm(Norm):
+    def tensor_decls(self) -> List[TensorDecl]:
+        decls = [TensorDecl(self.spec.weight, (self.width,), FLOAT32, init="gain")]
+        if self.spec.bias is not None:
+            decls.append(TensorDecl(self.spec.bias, (self.width,), FLOAT32, init="bias"))
+        return decls
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        self.gain = weights[self.spec.weight]
+        self.bias = weights[self.spec.bias] if self.spec.bias is not None else None
+
+    def small_tensors(self):
+        return [t for t in (self.gain, self.bias) if t is not None]
+
+    def emit(self, plan) -> int:
+        return plan.layer_norm(self.gain, self.bias, self.spec.eps)
