@@ -303,6 +303,31 @@ def lfm2_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
                 block_auto_adjust_ff_dim=False, vocab_size=vocab, tie_embedding=False)
 
 
+def rukosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Rukosun model of `layers` layers (the two latent-attention kinds in turn) whose sizes resemble a real model's
+    at this width: heads of 64 (32 unrotated, 32 rotated), values of 64, a cached row of 96 + 32 values per token and
+    layer, queries through a latent of half the width, windows of 1,024 and 512, four residual streams."""
+    heads = width // 64
+    first = {"heads": heads, "dim": 32, "rot_dim": 32, "vdim": 64, "kv_rank": 96, "q_rank": width // 2, "scale": 0.125,
+             "rot": {"base": 10000.0, "dims": 32}, "mask": {"size": 1024}}
+    second = {k: v for k, v in first.items() if k != "q_rank"}
+    second["mask"] = {"size": 512}
+    kinds = [{"type": "latent_attention", "mixer": first}, {"type": "latent_attention_2", "mixer": second}]
+    mlp = {"kind": "dense", "ff": ff}
+    return {"architecture": "Rukosun", "vocab": vocab, "width": width, "max_positions": 8192, "norm": {"eps": 1e-6}, "streams": 4,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "layers": [dict(kinds[i % 2], mlp=mlp) for i in range(layers)]}
+
+
+def lfm2_attention_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """The closest model the framework had to a decoder of attention layers only: LFM2 at the same width, feed-forward,
+    depth and vocabulary with every layer an attention layer (heads of 64 in groups of four)."""
+    return dict(lfm2_shape(width, ff, layers, vocab), full_attn_idxs=list(range(layers)))
+
+
+BESIDE = {"zokepel": ("Zokepel", zokepel_shape, lfm2_shape), "rukosun": ("Rukosun", rukosun_shape, lfm2_attention_shape)}
+
+
 def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
     import torch
 
@@ -318,8 +343,9 @@ def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
 
 
 def compare_designs(args) -> int:
-    """`--design zokepel`: prefill and decode speed of Zokepel at a few sizes beside LFM2 at equal width, depth,
-    feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One JSON line."""
+    """`--design zokepel` / `--design rukosun`: prefill and decode speed of that design at a few sizes beside LFM2 at equal
+    width, depth, feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One
+    JSON line."""
     import gc
 
     import torch
@@ -328,10 +354,13 @@ def compare_designs(args) -> int:
     sizes = {"small": [(1024, 4096, 6, 32768)], "medium": [(2048, 8192, 6, 65536)],
              "all": [(1024, 4096, 6, 32768), (2048, 8192, 6, 65536), (4096, 12288, 3, 65536)]}[args.sizes]
     rows = []
+    name, its_shape, lfm2_beside = BESIDE[args.design]
     for width, ff, layers, vocab in sizes:
-        for design, shape in (("Zokepel", zokepel_shape(width, ff, layers, vocab)), ("LFM2", lfm2_shape(width, ff, layers, vocab))):
+        for design, shape in ((name, its_shape(width, ff, layers, vocab)), ("LFM2", lfm2_beside(width, ff, layers, vocab))):
+            print(f"[bench] {design} width {width}: building", file=sys.stderr, flush=True)
             engine = engine_of(shape, args.dtype, max_requests=args.batch, context=4096)
             row = {"design": design, "width": width, "ff": ff, "layers": layers, "vocab": vocab}
+            print(f"[bench] {design} width {width}: prompt", file=sys.stderr, flush=True)
             prefill_s = time_prefill(engine, n_tokens=args.prefill_tokens)
             row["prefill_tok_s"] = round(args.prefill_tokens / prefill_s, 1)
             row["prefill_ms"] = round(prefill_s * 1e3, 3)
@@ -339,6 +368,7 @@ def compare_designs(args) -> int:
             if not args.no_kernels:
                 ids = seeded_prompt(5, args.prefill_tokens, vocab)
                 row["prefill_kernels"] = kernel_shares(lambda: (engine.step([("k", ids, [len(ids) - 1])]), engine.release("k")), most=10)
+            print(f"[bench] {design} width {width}: decode", file=sys.stderr, flush=True)
             dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels, prompt_len=args.prompt_len)
             row["decode_tok_s"] = round(args.batch * args.steps / dt, 1)
             row["decode_ms_per_step"] = round(dt / args.steps * 1e3, 4)
@@ -355,9 +385,9 @@ def compare_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["lfm2", "zokepel"], default="lfm2",
-                    help="zokepel: that design beside LFM2 at equal sizes instead of the headline workload")
-    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel")
+    ap.add_argument("--design", choices=["lfm2", "zokepel", "rukosun"], default="lfm2",
+                    help="zokepel, rukosun: that design beside LFM2 at equal sizes instead of the headline workload")
+    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel / rukosun")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -385,7 +415,7 @@ def main() -> int:
         print(f"--prompt-len + --warmup + {RUNS + 1} x --steps must stay below the context ({context})")
         return 2
 
-    if args.design == "zokepel":
+    if args.design in BESIDE:
         return compare_designs(args)
     from gibbs_amd import roofline as R
     gate = None if args.no_parity else parity()

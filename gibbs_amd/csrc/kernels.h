@@ -41,16 +41,22 @@ int gibbs_streams_norm(const float* x, int streams, long stream_stride, const fl
                        hipStream_t stream);
 int gibbs_streams_write(float* x, int streams, long stream_stride, const float* mix, const float* out_coef, const void* delta,
                         int delta_dtype, int parts, long part_stride, long count, hipStream_t stream);
+int gibbs_streams_write_norm(float* x, int streams, long stream_stride, const float* mix, const float* out_coef,
+                             const void* delta, int delta_dtype, int parts, long part_stride, int n_rows, int hidden,
+                             const float* coef, int kind, const float* gain, const float* bias, float eps, void* out, int dtype,
+                             hipStream_t stream);
 int gibbs_rms_rows_ld(const void* in, long ld_in, const float* gain, float eps, void* out, long ld_out, int dtype, int n,
                       int width, hipStream_t stream);
 int gibbs_latent_prepare(const void* kv, long ld_kv, const void* q, long ld_q, void* q_out, long ld_qo, void* pages, int dtype,
                          const float* gain, float eps, const float* inv_freq, int rot_dims, int variant, const int* pos,
                          const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh,
                          int dim, int rot, int rank, hipStream_t stream);
-int gibbs_sigmoid_gate(void* o, long ld_o, const void* g, long ld_g, int dtype, int n, int width, hipStream_t stream);
 int gibbs_poly_norm(const void* z, void* out, int dtype, const float* coef, float eps, int n, int F, hipStream_t stream);
 int gibbs_gemm_heads(const void* X, long ldx, long head_x, const void* W, long head_w, long ldw, void* Y, long ldy, long head_y,
                      int dtype, int n, int O, int I, int heads, hipStream_t stream);
+int gibbs_gemm_heads_gated(const void* X, long ldx, long head_x, const void* W, long head_w, long ldw, void* Y, long ldy,
+                           long head_y, const void* G, long ldg, long head_g, int dtype, int n, int O, int I, int heads,
+                           hipStream_t stream);
 int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype, const int* pos, const int* row_req,
                      const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
                      float eps, int unit, int norm_dim, float temp_coef, int temp_every, hipStream_t stream);

@@ -267,6 +267,8 @@ struct NormPart {
   // the norm of a weighted sum of several residual streams x [streams][N][hidden] (coef null: their plain sum), of all
   // rows or of `rows`; the streams are not touched
   virtual void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const;
+  // a norm that the streams' kernels apply themselves: its kind there (0 root mean square, 1 layer norm) and operands
+  virtual bool for_streams(int* kind, const float** gain, const float** bias, float* eps) const { return false; }
 };
 
 struct Body {
@@ -391,6 +393,10 @@ struct RmsNorm : NormPart {
     RUN(e, gibbs_streams_norm(x, streams, (long)e.a.n_rows * H, coef, 0, gain, nullptr, eps, out, e.p.dtype, rows, n_out, H, e.a.stream));
     return out;
   }
+  bool for_streams(int* kind, const float** g, const float** b, float* e) const override {
+    *kind = 0; *g = gain; *b = nullptr; *e = eps;
+    return true;
+  }
   void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const override {
     const int H = e.p.hidden;
     void* out = e.take((long)n_out * H * e.esize);
@@ -435,6 +441,10 @@ struct LayerNorm : NormPart {
   void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const override {
     e.settle(x, pending);
     return run_streams(e, x, 1, nullptr, rows, n_out);
+  }
+  bool for_streams(int* kind, const float** g, const float** b, float* e) const override {
+    *kind = 1; *g = gain; *b = bias; *e = eps;
+    return true;
   }
 };
 struct HostNorm : NormPart {
@@ -842,9 +852,10 @@ struct LatentBody : Body {
     void* att = attend_prepared(e, t, q_lat, (long)H * L, (long)H * L);
     e.give(q_lat);
     void* o = e.take((long)N * H * V * e.esize);
-    RUN(e, gibbs_gemm_heads(att, (long)H * L, L, uv, (long)V * C, C, o, (long)H * V, V, e.p.dtype, N, V, C, H, a.stream));
+    // (the gate multiplies the values' up-projection as it is stored)
+    RUN(e, gibbs_gemm_heads_gated(att, (long)H * L, L, uv, (long)V * C, C, o, (long)H * V, V, off_g >= 0 ? raw + (long)off_g * e.esize : nullptr,
+                                  in.O, V, e.p.dtype, N, V, C, H, a.stream));
     e.give(att);
-    if (off_g >= 0) RUN(e, gibbs_sigmoid_gate(o, (long)H * V, raw + (long)off_g * e.esize, in.O, e.p.dtype, N, H * V, a.stream));
     e.give(raw);
     Pending delta;
     delta.data = e.linear(o, out, N, false, true, true, &delta.parts);
@@ -974,12 +985,25 @@ void Exec::run() {
         rows[op.result] = p.norms[op.norm]->run_streams(*this, x, S, p.hypers[op.body].in, nullptr, N);
         break;
       case Plan::OP_STREAMS_ADD: {
+        // the streams are written and, where the next operation reads them for a norm that the kernel knows, read in the
+        // same pass (the rows are in registers already: a sublayer's boundary is one kernel, not two)
         const Hyper& hc = p.hypers[op.body];
         Pending& d = deltas[op.value];
-        RUN(*this, gibbs_streams_write(x, S, (long)N * H, hc.mix, hc.out, d.data, d.parts >= 2 ? GIBBS_F32 : p.dtype, std::max(d.parts, 1),
-                                       (long)N * H, (long)N * H, a.stream));
+        const Plan::Op* next = i + 1 < last && p.ops[i + 1].kind == Plan::OP_STREAMS_NORM ? &p.ops[i + 1] : nullptr;
+        int kind = 0;
+        const float *gain = nullptr, *bias = nullptr;
+        float eps = 0.f;
+        if (next && !p.norms[next->norm]->for_streams(&kind, &gain, &bias, &eps)) next = nullptr;
+        void* out = next ? take((long)N * H * esize) : nullptr;
+        RUN(*this, gibbs_streams_write_norm(x, S, (long)N * H, hc.mix, hc.out, d.data, d.parts >= 2 ? GIBBS_F32 : p.dtype, std::max(d.parts, 1),
+                                            (long)N * H, N, H, next ? p.hypers[next->body].in : nullptr, kind, gain, bias, eps, out, p.dtype,
+                                            a.stream));
         give(d.data);
         d = Pending{};
+        if (next) {
+          rows[next->result] = out;
+          ++i;
+        }
         break;
       }
       case Plan::OP_DROP:

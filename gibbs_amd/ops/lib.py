@@ -72,14 +72,17 @@ _SIGNATURES = {
     "gibbs_streams_norm": [c_void_p, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_int,
                            c_int, c_void_p],
     "gibbs_streams_write": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_void_p],
+    "gibbs_streams_write_norm": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_void_p,
+                                 c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p],
     "gibbs_rms_rows_ld": [c_void_p, c_long, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
     "gibbs_latent_prepare": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_float, c_void_p,
                              c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                              c_void_p],
-    "gibbs_sigmoid_gate": [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
     "gibbs_poly_norm": [c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p],
     "gibbs_gemm_heads": [c_void_p, c_long, c_long, c_void_p, c_long, c_long, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int,
                          c_int, c_void_p],
+    "gibbs_gemm_heads_gated": [c_void_p, c_long, c_long, c_void_p, c_long, c_long, c_void_p, c_long, c_long, c_void_p, c_long, c_long,
+                               c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_qk_unit_kv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_int, c_void_p],
     "gibbs_causal_conv_silu": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
