@@ -346,11 +346,28 @@ def compare_designs(args) -> int:
     """`--design zokepel` / `--design rukosun`: prefill and decode speed of that design at a few sizes beside LFM2 at equal
     width, depth, feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One
     JSON line."""
+    import faulthandler
     import gc
 
     import torch
 
     from gibbs_amd import roofline as R
+    faulthandler.enable()       # (a crash inside a library names the Python frame it came from)
+    # The kernels' shares come from the profiler, which sometimes dies when it stops after replays of captured
+    # graphs; they are therefore measured by a child process of their own, first, and a child that fails costs
+    # the listing only.  This process then measures the times with no profiler loaded.
+    listed = {}
+    if not args.no_kernels and not args.kernels_child:
+        import subprocess
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--design", args.design, "--sizes", args.sizes, "--kernels-child",
+                                "--dtype", args.dtype, "--batch", str(args.batch), "--prompt-len", str(args.prompt_len),
+                                "--prefill-tokens", str(args.prefill_tokens), "--steps", str(args.steps), "--warmup", str(args.warmup)],
+                               stdout=subprocess.PIPE, text=True)
+        if child.returncode == 0:
+            listed = {(r["design"], r["width"]): r for r in json.loads(child.stdout.strip().splitlines()[-1])["rows"]}
+        else:
+            print(f"[bench] the kernels' shares were not measured (the profiling process ended with {child.returncode})", file=sys.stderr, flush=True)
+    profile = bool(args.kernels_child)
     sizes = {"small": [(1024, 4096, 6, 32768)], "medium": [(2048, 8192, 6, 65536)],
              "all": [(1024, 4096, 6, 32768), (2048, 8192, 6, 65536), (4096, 12288, 3, 65536)]}[args.sizes]
     rows = []
@@ -365,15 +382,18 @@ def compare_designs(args) -> int:
             row["prefill_tok_s"] = round(args.prefill_tokens / prefill_s, 1)
             row["prefill_ms"] = round(prefill_s * 1e3, 3)
             row["prefill_frac_of_peak"] = round(R.prefill_flops(engine, args.prefill_tokens) / prefill_s / R.PEAK_FLOPS[args.dtype], 4)
-            if not args.no_kernels:
+            if profile:
                 ids = seeded_prompt(5, args.prefill_tokens, vocab)
                 row["prefill_kernels"] = kernel_shares(lambda: (engine.step([("k", ids, [len(ids) - 1])]), engine.release("k")), most=10)
             print(f"[bench] {design} width {width}: decode", file=sys.stderr, flush=True)
-            dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels, prompt_len=args.prompt_len)
+            dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=profile, prompt_len=args.prompt_len)
             row["decode_tok_s"] = round(args.batch * args.steps / dt, 1)
             row["decode_ms_per_step"] = round(dt / args.steps * 1e3, 4)
             row["decode_frac_of_hbm"] = round(R.decode_bytes(engine, seq_lens) / (dt / args.steps) / R.HBM_BYTES_PER_S, 4)
             row["decode_kernels"] = top
+            if (design, width) in listed:
+                row["prefill_kernels"] = listed[(design, width)].get("prefill_kernels")
+                row["decode_kernels"] = listed[(design, width)].get("decode_kernels")
             rows.append(row)
             del engine
             gc.collect()
@@ -402,6 +422,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate")
     ap.add_argument("--no-kernels", action="store_true", help="skip the kernels' shares of the decode step")
+    ap.add_argument("--kernels-child", action="store_true", help=argparse.SUPPRESS)    # (the profiling process of a design comparison)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (this engine has no multi-GPU path); got --gpus {args.gpus}")

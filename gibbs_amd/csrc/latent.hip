@@ -5,53 +5,9 @@
 //
 // Sums, norms, angles and the streams themselves are float32 whatever the run's activation type is.
 #include "common.h"
+#include <algorithm>
 
 namespace {
-// ------------------------------------------------------------------------------------------------- embedding
-// x[c][n][:] = table[id] + pair_table[row] + pos_table[pos], c = 0 .. copies - 1, with
-//   row = buckets                                  for a sequence's first token (position 0)
-//         (prev * mul_prev + id * mul_cur) mod buckets   otherwise,
-// prev being the row before in this step, or, for the first row of a request's portion, the token that the
-// request's state slot holds (what gibbs_store_last_token left there).
-template <typename T>
-__global__ void embed_tables_kernel(const T* __restrict__ table, const T* __restrict__ pair_table, const T* __restrict__ pos_table,
-                                    const int* __restrict__ ids, const int* __restrict__ pos, const int* __restrict__ row_req,
-                                    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ prev,
-                                    long slot_stride, float* __restrict__ x, int copies, int n_rows, int hidden, int vocab,
-                                    int buckets, int mul_prev, int mul_cur, int pos_len) {
-  const int n = blockIdx.x;
-  int id = ids[n];
-  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);      // (never read outside the table)
-  const T* row = table + (size_t)id * hidden;
-  const T* pair = nullptr;
-  const int p = pos[n];
-  if (pair_table) {
-    long r = buckets;
-    if (p > 0) {
-      const int req = row_req[n];
-      int before = n > cu[req] ? ids[n - 1] : prev[(size_t)slot[req] * slot_stride];
-      before = before < 0 ? 0 : (before >= vocab ? vocab - 1 : before);
-      r = ((long)before * mul_prev + (long)id * mul_cur) % buckets;
-    }
-    pair = pair_table + (size_t)r * hidden;
-  }
-  const T* at = pos_table ? pos_table + (size_t)min(max(p, 0), pos_len - 1) * hidden : nullptr;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float v = to_float(row[i]);
-    if (pair) v += to_float(pair[i]);
-    if (at) v += to_float(at[i]);
-    for (int c = 0; c < copies; ++c) x[((size_t)c * n_rows + n) * hidden + i] = v;
-  }
-}
-
-__global__ void store_last_token_kernel(const int* __restrict__ ids, const int* __restrict__ cu, const int* __restrict__ slot,
-                                        int* __restrict__ prev, long slot_stride, int n_req) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= n_req || cu[r + 1] <= cu[r]) return;
-  prev[(size_t)slot[r] * slot_stride] = ids[cu[r + 1] - 1];
-}
-
-// ------------------------------------------------------------------------------------------------- streams
 // Elements a thread takes at a time: four floats (or bfloat16 values) where rows allow it, else one.
 template <int V> struct FloatVec { float v[V]; };
 template <int V> __device__ __forceinline__ FloatVec<V> load_vec(const float* p) {
@@ -85,6 +41,66 @@ template <int V> __device__ __forceinline__ void store_vec(bf16* p, const FloatV
   }
 }
 
+// Threads of a workgroup that owns a row of `per` vectors: few rows get wide workgroups (one pass over the row, every load in
+// flight at once: such a step is a chain of short kernels that wait for memory), many rows get 256 threads.
+int row_threads(int per, int n_rows) {
+  if (n_rows <= 256 && per > 256) return std::min(1024, (per + 63) / 64 * 64);
+  return per >= 512 ? 256 : (per >= 128 ? 128 : 64);
+}
+
+// ------------------------------------------------------------------------------------------------- embedding
+// x[c][n][:] = table[id] + pair_table[row] + pos_table[pos], c = 0 .. copies - 1, with
+//   row = buckets                                  for a sequence's first token (position 0)
+//         (prev * mul_prev + id * mul_cur) mod buckets   otherwise,
+// prev being the row before in this step, or, for the first row of a request's portion, the token that the
+// request's state slot holds (what gibbs_store_last_token left there).
+template <typename T, int V>
+__global__ void embed_tables_kernel(const T* __restrict__ table, const T* __restrict__ pair_table, const T* __restrict__ pos_table,
+                                    const int* __restrict__ ids, const int* __restrict__ pos, const int* __restrict__ row_req,
+                                    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ prev,
+                                    long slot_stride, float* __restrict__ x, int copies, int n_rows, int hidden, int vocab,
+                                    int buckets, int mul_prev, int mul_cur, int pos_len) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);      // (never read outside the table)
+  const T* row = table + (size_t)id * hidden;
+  const T* pair = nullptr;
+  const int p = pos[n];
+  if (pair_table) {
+    long r = buckets;
+    if (p > 0) {
+      const int req = row_req[n];
+      int before = n > cu[req] ? ids[n - 1] : prev[(size_t)slot[req] * slot_stride];
+      before = before < 0 ? 0 : (before >= vocab ? vocab - 1 : before);
+      r = ((long)before * mul_prev + (long)id * mul_cur) % buckets;
+    }
+    pair = pair_table + (size_t)r * hidden;
+  }
+  const T* at = pos_table ? pos_table + (size_t)min(max(p, 0), pos_len - 1) * hidden : nullptr;
+  for (int i = threadIdx.x * V; i < hidden; i += blockDim.x * V) {
+    FloatVec<V> v = load_vec<V>(row + i);
+    if (pair) {
+      const FloatVec<V> more = load_vec<V>(pair + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) v.v[e] += more.v[e];
+    }
+    if (at) {
+      const FloatVec<V> more = load_vec<V>(at + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) v.v[e] += more.v[e];
+    }
+    for (int c = 0; c < copies; ++c) store_vec<V>(x + ((size_t)c * n_rows + n) * hidden + i, v);
+  }
+}
+
+__global__ void store_last_token_kernel(const int* __restrict__ ids, const int* __restrict__ cu, const int* __restrict__ slot,
+                                        int* __restrict__ prev, long slot_stride, int n_req) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_req || cu[r + 1] <= cu[r]) return;
+  prev[(size_t)slot[r] * slot_stride] = ids[cu[r + 1] - 1];
+}
+
+// ------------------------------------------------------------------------------------------------- streams
 // One workgroup per row.  WRITE: first all streams are written at once from the old ones,
 //   x[t] <- sum_s mix[s][t] x[s] + out_coef[t] * y, s ascending, y the delta (one part in its type, or float32 partial
 //   sums added in ascending order);
@@ -184,20 +200,27 @@ __global__ void streams_kernel(float* __restrict__ x, long stream_stride, const 
 }
 
 // ------------------------------------------------------------------------------------------------- rows
-// out[n][:] = in[n][:width] / sqrt(mean(in^2) + eps) * gain; one wave per row.
-template <typename T>
+// out[n][:] = in[n][:width] / sqrt(mean(in^2) + eps) * gain; one workgroup per row, V values a thread at a time.
+template <typename T, int V>
 __global__ void rms_rows_ld_kernel(const T* __restrict__ in, long ld_in, const float* __restrict__ gain, float eps,
-                                   T* __restrict__ out, long ld_out, int n, int width) {
-  const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  if (row >= n) return;
-  const T* src = in + (size_t)row * ld_in;
+                                   T* __restrict__ out, long ld_out, int width) {
+  __shared__ float scratch[16];
+  const T* src = in + (size_t)blockIdx.x * ld_in;
   float sq = 0.f;
-  for (int i = lane; i < width; i += WAVE) {
-    const float v = to_float(src[i]);
-    sq = fmaf(v, v, sq);
+#pragma unroll 4
+  for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+    const FloatVec<V> r = load_vec<V>(src + i);
+#pragma unroll
+    for (int e = 0; e < V; ++e) sq = fmaf(r.v[e], r.v[e], sq);
   }
-  const float r = 1.0f / sqrtf(wave_sum(sq) / (float)width + eps);
-  for (int i = lane; i < width; i += WAVE) out[(size_t)row * ld_out + i] = from_float<T>(to_float(src[i]) * r * (gain ? gain[i] : 1.f));
+  const float r = 1.0f / sqrtf(block_sum(sq, scratch) / (float)width + eps);
+#pragma unroll 4
+  for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+    FloatVec<V> o = load_vec<V>(src + i);
+#pragma unroll
+    for (int e = 0; e < V; ++e) o.v[e] = o.v[e] * r * (gain ? gain[i + e] : 1.f);
+    store_vec<V>(out + (size_t)blockIdx.x * ld_out + i, o);
+  }
 }
 
 // The pair (u, v) at position p becomes (u cos a - v sin a, v cos a + u sin a), a = float(p) * inv_freq[i].
@@ -424,17 +447,20 @@ GIBBS_EXPORT int gibbs_embed_tables(const void* table, const void* pair_table, c
   GIBBS_REQUIRE(!pair_table || (buckets > 0 && row_req && cu && slot && prev), "embed_tables: the pair table needs its buckets, the batch's layout and the requests' last tokens");
   GIBBS_REQUIRE(!pos_table || pos_len > 0, "embed_tables: an empty position table");
   if (n == 0) return 0;
-  const int threads = hidden >= 1024 ? 256 : 64;
-  if (dtype == GIBBS_F32)
-    embed_tables_kernel<float><<<n, threads, 0, stream>>>((const float*)table, (const float*)pair_table, (const float*)pos_table, ids, pos,
-                                                          row_req, cu, slot, prev, slot_stride, x, copies, n, hidden, vocab, buckets,
-                                                          mul_prev, mul_cur, pos_len);
-  else if (dtype == GIBBS_BF16)
-    embed_tables_kernel<bf16><<<n, threads, 0, stream>>>((const bf16*)table, (const bf16*)pair_table, (const bf16*)pos_table, ids, pos,
-                                                         row_req, cu, slot, prev, slot_stride, x, copies, n, hidden, vocab, buckets,
-                                                         mul_prev, mul_cur, pos_len);
-  else
+  const bool vec = hidden % 4 == 0 && ((uintptr_t)table % 16) == 0 && ((uintptr_t)pair_table % 16) == 0 && ((uintptr_t)pos_table % 16) == 0 &&
+                   ((uintptr_t)x % 16) == 0;
+  const int threads = row_threads(vec ? hidden / 4 : hidden, n);
+#define GIBBS_EMBED(T, V)                                                                                                        \
+  embed_tables_kernel<T, V><<<n, threads, 0, stream>>>((const T*)table, (const T*)pair_table, (const T*)pos_table, ids, pos, row_req, cu, \
+                                                       slot, prev, slot_stride, x, copies, n, hidden, vocab, buckets, mul_prev, mul_cur, pos_len)
+  if (dtype == GIBBS_F32) {
+    if (vec) GIBBS_EMBED(float, 4); else GIBBS_EMBED(float, 1);
+  } else if (dtype == GIBBS_BF16) {
+    if (vec) GIBBS_EMBED(bf16, 4); else GIBBS_EMBED(bf16, 1);
+  } else {
     return gibbs_fail("embed_tables: unknown dtype %d", dtype);
+  }
+#undef GIBBS_EMBED
   GIBBS_LAUNCH_STATUS("embed_tables");
 }
 
@@ -452,8 +478,7 @@ template <int S, int V, typename T, typename TD, bool WRITE, bool NORM>
 void launch_streams_one(int n_rows, int hidden, hipStream_t stream, float* x, long stream_stride, const float* mix, const float* out_coef,
                         const TD* delta, int parts, long part_stride, const float* coef, int kind, const float* gain, const float* bias,
                         float eps, T* out, const int* rows) {
-  const int per = hidden / V;
-  const int threads = per >= 512 ? 256 : (per >= 128 ? 128 : 64);
+  const int threads = row_threads(hidden / V, n_rows);
   streams_kernel<S, V, T, TD, WRITE, NORM><<<n_rows, threads, NORM ? (size_t)hidden * 4 : 0, stream>>>(
       x, stream_stride, mix, out_coef, delta, parts, part_stride, coef, kind, gain, bias, eps, out, rows, hidden);
 }
@@ -539,13 +564,17 @@ GIBBS_EXPORT int gibbs_streams_write(float* x, int streams, long stream_stride, 
 GIBBS_EXPORT int gibbs_rms_rows_ld(const void* in, long ld_in, const float* gain, float eps, void* out, long ld_out, int dtype, int n,
                                    int width, hipStream_t stream) {
   GIBBS_REQUIRE(n >= 0 && width > 0 && ld_in >= width && ld_out >= width, "rms_rows: bad sizes n=%d width=%d", n, width);
+  GIBBS_REQUIRE(dtype == GIBBS_F32 || dtype == GIBBS_BF16, "rms_rows: unknown dtype %d", dtype);
   if (n == 0) return 0;
-  if (dtype == GIBBS_F32)
-    rms_rows_ld_kernel<float><<<ceil_div(n, 4), 256, 0, stream>>>((const float*)in, ld_in, gain, eps, (float*)out, ld_out, n, width);
-  else if (dtype == GIBBS_BF16)
-    rms_rows_ld_kernel<bf16><<<ceil_div(n, 4), 256, 0, stream>>>((const bf16*)in, ld_in, gain, eps, (bf16*)out, ld_out, n, width);
-  else
-    return gibbs_fail("rms_rows: unknown dtype %d", dtype);
+  const bool vec = width % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int threads = row_threads(vec ? width / 4 : width, n);
+  if (dtype == GIBBS_F32) {
+    if (vec) rms_rows_ld_kernel<float, 4><<<n, threads, 0, stream>>>((const float*)in, ld_in, gain, eps, (float*)out, ld_out, width);
+    else rms_rows_ld_kernel<float, 1><<<n, threads, 0, stream>>>((const float*)in, ld_in, gain, eps, (float*)out, ld_out, width);
+  } else {
+    if (vec) rms_rows_ld_kernel<bf16, 4><<<n, threads, 0, stream>>>((const bf16*)in, ld_in, gain, eps, (bf16*)out, ld_out, width);
+    else rms_rows_ld_kernel<bf16, 1><<<n, threads, 0, stream>>>((const bf16*)in, ld_in, gain, eps, (bf16*)out, ld_out, width);
+  }
   GIBBS_LAUNCH_STATUS("rms_rows");
 }
 
@@ -582,8 +611,7 @@ GIBBS_EXPORT int gibbs_poly_norm(const void* z, void* out, int dtype, const floa
   if (n == 0) return 0;
   const bool vec = F % 4 == 0 && ((uintptr_t)z % 16) == 0 && ((uintptr_t)out % 16) == 0;
   const bool keep = F <= 16000;
-  const int per = vec ? F / 4 : F;
-  const int threads = per >= 512 ? 256 : (per >= 128 ? 128 : 64);
+  const int threads = row_threads(vec ? F / 4 : F, n);
   const size_t lds = keep ? (size_t)F * 4 : 0;
 #define GIBBS_POLY(T, V, KEEP) poly_norm_kernel<T, V, KEEP><<<n, threads, lds, stream>>>((const T*)z, (T*)out, coef, eps, F)
   if (dtype == GIBBS_F32) {
