@@ -291,44 +291,77 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const T* __restrict
 }
 
 // out = a N(z) + b N(z^2) + c N(z^3) + e over a row of F values, N(v) = v / sqrt(mean(v^2) + eps), powers element by element.
-// One workgroup per row; the row is read once, V values a thread at a time, and kept in LDS (F floats) when KEEP.
-template <typename T, int V, bool KEEP>
+// One workgroup per row; the row is read once, V values a thread at a time, and kept between the sums and the result:
+// KEEP 2 in registers (up to 8 vectors a thread, all loads in flight at once), KEEP 1 in LDS (F floats), KEEP 0 read again.
+template <typename T, int V, int KEEP>
 __global__ void poly_norm_kernel(const T* __restrict__ z, T* __restrict__ out, const float* __restrict__ coef, float eps, int F) {
   extern __shared__ float kept[];
   __shared__ float scratch[16];
   const T* src = z + (size_t)blockIdx.x * F;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-#pragma unroll 4
-  for (int i = threadIdx.x * V; i < F; i += blockDim.x * V) {
-    const FloatVec<V> r = load_vec<V>(src + i);
+  FloatVec<V> mine[KEEP == 2 ? 8 : 1];
+  if constexpr (KEEP == 2) {
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const float v = r.v[e], v2 = v * v;
-      if constexpr (KEEP) kept[i + e] = v;
-      s2 += v2;
-      s4 = fmaf(v2, v2, s4);
-      s6 = fmaf(v2 * v, v2 * v, s6);
+    for (int j = 0; j < 8; ++j) {
+      const int i = (threadIdx.x + j * blockDim.x) * V;
+      if (i < F) mine[j] = load_vec<V>(src + i);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = (threadIdx.x + j * blockDim.x) * V;
+      if (i >= F) continue;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float v = mine[j].v[e], v2 = v * v;
+        s2 += v2;
+        s4 = fmaf(v2, v2, s4);
+        s6 = fmaf(v2 * v, v2 * v, s6);
+      }
+    }
+  } else {
+#pragma unroll 4
+    for (int i = threadIdx.x * V; i < F; i += blockDim.x * V) {
+      const FloatVec<V> r = load_vec<V>(src + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float v = r.v[e], v2 = v * v;
+        if constexpr (KEEP == 1) kept[i + e] = v;
+        s2 += v2;
+        s4 = fmaf(v2, v2, s4);
+        s6 = fmaf(v2 * v, v2 * v, s6);
+      }
     }
   }
   const float r1 = coef[0] / sqrtf(block_sum(s2, scratch) / (float)F + eps);
   const float r2 = coef[1] / sqrtf(block_sum(s4, scratch) / (float)F + eps);
   const float r3 = coef[2] / sqrtf(block_sum(s6, scratch) / (float)F + eps);
   const float c0 = coef[3];
-#pragma unroll 4
-  for (int i = threadIdx.x * V; i < F; i += blockDim.x * V) {
-    FloatVec<V> r;
-    if constexpr (KEEP) {
-#pragma unroll
-      for (int e = 0; e < V; ++e) r.v[e] = kept[i + e];
-    } else {
-      r = load_vec<V>(src + i);
-    }
+  auto result = [&](FloatVec<V> r) {
 #pragma unroll
     for (int e = 0; e < V; ++e) {
       const float v = r.v[e], v2 = v * v;
       r.v[e] = fmaf(r1, v, fmaf(r2, v2, fmaf(r3, v2 * v, c0)));
     }
-    store_vec<V>(out + (size_t)blockIdx.x * F + i, r);
+    return r;
+  };
+  if constexpr (KEEP == 2) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = (threadIdx.x + j * blockDim.x) * V;
+      if (i < F) store_vec<V>(out + (size_t)blockIdx.x * F + i, result(mine[j]));
+    }
+  } else {
+#pragma unroll 4
+    for (int i = threadIdx.x * V; i < F; i += blockDim.x * V) {
+      FloatVec<V> r;
+      if constexpr (KEEP == 1) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) r.v[e] = kept[i + e];
+      } else {
+        r = load_vec<V>(src + i);
+      }
+      store_vec<V>(out + (size_t)blockIdx.x * F + i, result(r));
+    }
   }
 }
 
@@ -393,9 +426,13 @@ __global__ __launch_bounds__(256) void gemm_heads_plain_kernel(const T* __restri
 // The same on the matrix cores, for bfloat16 slices whose rows start at multiples of 16 bytes and whose inner
 // size is a multiple of 8: a wave takes 16 rows x 64 features, four 16 x 16 x 32 products per step of k, both
 // operands straight from memory (X and W are contiguous along k, which is the operand layout: lane l holds
-// the 8 values k = (l / 16) * 8 .. + 8 of row or feature l % 16); a workgroup is 4 waves on 64 rows.
+// the 8 values k = (l / 16) * 8 .. + 8 of row or feature l % 16); a workgroup is 4 waves on 64 rows.  W is the
+// first operand (the tile is Y^T = W X^T), so a lane's four results are four neighbouring features of one row:
+// with VEC they leave (and the gate arrives) as one 8-byte access.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+template <bool VEC>
 __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(const bf16* __restrict__ X, long ldx, long head_x, const bf16* __restrict__ W,
                                                               long head_w, long ldw, bf16* __restrict__ Y, long ldy, long head_y, int N,
                                                               int O, int I, const bf16* __restrict__ G, long ldg, long head_g) {
@@ -403,6 +440,7 @@ __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(const bf16* __rest
   X += (size_t)h * head_x;
   W += (size_t)h * head_w;
   Y += (size_t)h * head_y;
+  if (G) G += (size_t)h * head_g;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int lr = lane % 16, lg = lane / 16;
   const int row = blockIdx.y * 64 + wave * 16 + lr;
@@ -414,25 +452,35 @@ __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(const bf16* __rest
   const bf16* xr = X + (size_t)min(row, N - 1) * ldx;
   for (int k0 = 0; k0 < I; k0 += 32) {
     const int k = k0 + lg * 8;
-    const bf16x8 a = (row < N && k < I) ? *(const bf16x8*)(xr + k) : zero8;
+    const bf16x8 x8 = (row < N && k < I) ? *(const bf16x8*)(xr + k) : zero8;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int col = col0 + t * 16 + lr;
-      const bf16x8 b = (col < O && k < I) ? *(const bf16x8*)(W + (size_t)col * ldw + k) : zero8;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+      const bf16x8 w8 = (col < O && k < I) ? *(const bf16x8*)(W + (size_t)col * ldw + k) : zero8;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w8, x8, acc[t], 0, 0, 0);
     }
   }
-  // element i of a lane's result: row (lane / 16) * 4 + i of the wave's 16, feature lane % 16 of the tile
+  // element i of a lane's result: feature (lane / 16) * 4 + i of the tile's 16, row lane % 16 of the wave's 16
+  if (row >= N) return;
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    const int col = col0 + t * 16 + lr;
+    const int col = col0 + t * 16 + lg * 4;
+    if (VEC && col + 4 <= O) {
+      float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+      if (G) {
+        const bf16x4 g4 = *(const bf16x4*)(G + (size_t)row * ldg + col);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] /= 1.0f + __expf(-(float)g4[i]);
+      }
+      *(bf16x4*)(Y + (size_t)row * ldy + col) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = blockIdx.y * 64 + wave * 16 + lg * 4 + i;
-      if (r >= N || col >= O) continue;
+      if (col + i >= O) continue;
       float v = acc[t][i];
-      if (G) v /= 1.0f + __expf(-(float)G[(size_t)r * ldg + (size_t)h * head_g + col]);
-      Y[(size_t)r * ldy + col] = (bf16)v;
+      if (G) v /= 1.0f + __expf(-(float)G[(size_t)row * ldg + col + i]);
+      Y[(size_t)row * ldy + col + i] = (bf16)v;
     }
   }
 }
@@ -610,16 +658,20 @@ GIBBS_EXPORT int gibbs_poly_norm(const void* z, void* out, int dtype, const floa
   GIBBS_REQUIRE(dtype == GIBBS_F32 || dtype == GIBBS_BF16, "poly_norm: unknown dtype %d", dtype);
   if (n == 0) return 0;
   const bool vec = F % 4 == 0 && ((uintptr_t)z % 16) == 0 && ((uintptr_t)out % 16) == 0;
-  const bool keep = F <= 16000;
-  const int threads = row_threads(vec ? F / 4 : F, n);
-  const size_t lds = keep ? (size_t)F * 4 : 0;
-#define GIBBS_POLY(T, V, KEEP) poly_norm_kernel<T, V, KEEP><<<n, threads, lds, stream>>>((const T*)z, (T*)out, coef, eps, F)
+  const int per = vec ? F / 4 : F;
+  const int threads = row_threads(per, n);
+  const int keep = per <= 8 * threads ? 2 : (F <= 16000 ? 1 : 0);
+  const size_t lds = keep == 1 ? (size_t)F * 4 : 0;
+#define GIBBS_POLY(T, V)                                                                                            \
+  do {                                                                                                              \
+    if (keep == 2) poly_norm_kernel<T, V, 2><<<n, threads, lds, stream>>>((const T*)z, (T*)out, coef, eps, F);      \
+    else if (keep == 1) poly_norm_kernel<T, V, 1><<<n, threads, lds, stream>>>((const T*)z, (T*)out, coef, eps, F); \
+    else poly_norm_kernel<T, V, 0><<<n, threads, lds, stream>>>((const T*)z, (T*)out, coef, eps, F);                \
+  } while (0)
   if (dtype == GIBBS_F32) {
-    if (vec && keep) GIBBS_POLY(float, 4, true); else if (vec) GIBBS_POLY(float, 4, false);
-    else if (keep) GIBBS_POLY(float, 1, true); else GIBBS_POLY(float, 1, false);
+    if (vec) GIBBS_POLY(float, 4); else GIBBS_POLY(float, 1);
   } else {
-    if (vec && keep) GIBBS_POLY(bf16, 4, true); else if (vec) GIBBS_POLY(bf16, 4, false);
-    else if (keep) GIBBS_POLY(bf16, 1, true); else GIBBS_POLY(bf16, 1, false);
+    if (vec) GIBBS_POLY(bf16, 4); else GIBBS_POLY(bf16, 1);
   }
 #undef GIBBS_POLY
   GIBBS_LAUNCH_STATUS("poly_norm");
@@ -644,8 +696,13 @@ GIBBS_EXPORT int gibbs_gemm_heads_gated(const void* X, long ldx, long head_x, co
   } else if (dtype == GIBBS_BF16) {
     const bool aligned = I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && head_x % 8 == 0 && head_w % 8 == 0 && ((uintptr_t)X % 16) == 0 &&
                          ((uintptr_t)W % 16) == 0;
-    if (aligned)
-      gemm_heads_mfma_kernel<<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I, (const bf16*)G, ldg, head_g);
+    // (8-byte stores and gate loads: rows, heads and the pointers themselves at multiples of 4 values)
+    const bool vec = ldy % 4 == 0 && head_y % 4 == 0 && ((uintptr_t)Y % 8) == 0 &&
+                     (!G || (ldg % 4 == 0 && head_g % 4 == 0 && ((uintptr_t)G % 8) == 0));
+    if (aligned && vec)
+      gemm_heads_mfma_kernel<true><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I, (const bf16*)G, ldg, head_g);
+    else if (aligned)
+      gemm_heads_mfma_kernel<false><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I, (const bf16*)G, ldg, head_g);
     else
       gemm_heads_plain_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, head_x, (const bf16*)W, head_w, ldw, (bf16*)Y, ldy, head_y, n, O, I, (const bf16*)G, ldg, head_g);
   } else {
