@@ -819,7 +819,7 @@ struct LatentBody : Body {
   Matrix in, uq, out;                 // uq.w null: queries come straight from `in`
   const void* uk_t = nullptr;         // [heads][rank][dim]: W_uk of every head, transposed
   const void* uv = nullptr;           // [heads][vdim][rank]
-  const float* q_gain = nullptr;      // [q_rank]
+  const float* q_gain = nullptr;      // [q_rank], or null: folded into W_uq's columns
   const float* kv_gain = nullptr;     // [rank]
   const float* sink = nullptr;        // [heads] or null
   const float* inv_freq = nullptr;    // [rot_dims / 2]
@@ -835,7 +835,13 @@ struct LatentBody : Body {
     char* raw = (char*)e.linear(h, in, N, false, false, false, nullptr);
     void* q = raw;
     long ld_q = in.O;
-    if (uq.w) {
+    if (uq.w && e.few_rows && !q_gain && q_rank % 8 == 0 && in.O % 8 == 0 && ((uintptr_t)raw % 16) == 0 && ((uintptr_t)uq.w % 16) == 0) {
+      // few rows, the latent's gain folded into W_uq: the product divides by the root mean square of the rows it reads
+      // (the few-row kernel's prologue, as in the other models' fused decode products)
+      q = e.take((long)N * uq.O * 2);
+      RUN(e, gibbs_skinny_store(raw, uq.w, q, N, uq.O, q_rank, in.O, q_rank, uq.O, 1, eps, a.stream));
+      ld_q = uq.O;
+    } else if (uq.w) {
       void* cq = e.take((long)N * q_rank * e.esize);
       RUN(e, gibbs_rms_rows_ld(raw, in.O, q_gain, eps, cq, q_rank, e.p.dtype, N, q_rank, a.stream));
       q = e.linear(cq, uq, N, false, false, false, nullptr);

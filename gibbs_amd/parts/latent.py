@@ -97,6 +97,11 @@ class LatentAttentionMixer(Mixer):
         self.off_g = offsets[2] if self.gate else -1
         self.w_uq = weights[t["uq"]] if self.q_rank else None
         self.q_gain = weights[t["dq_norm"]] if self.q_rank else None
+        if self.q_rank and rt.act_dtype == torch.bfloat16 and rt.fold_gains:
+            # the queries' latent is read by W_uq alone: its norm's gain goes into that matrix's columns (as the layer
+            # norms' gains of the other models do), and steps of few rows take the product that norms its rows itself
+            self.w_uq = (self.w_uq.float() * self.q_gain[None, :]).to(self.w_uq.dtype)
+            self.q_gain = None
         self.kv_gain = weights[t["dkv_norm"]]
         # every head's key up-projection transposed, [heads, kv_rank, dim]: the product that takes a head's unrotated
         # query part to the latent's size reads it as a matrix [out, in]
