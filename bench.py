@@ -315,7 +315,7 @@ def rukosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     kinds = [{"type": "latent_attention", "mixer": first}, {"type": "latent_attention_2", "mixer": second}]
     mlp = {"kind": "dense", "ff": ff}
     return {"architecture": "Rukosun", "vocab": vocab, "width": width, "max_positions": 8192, "norm": {"eps": 1e-6}, "streams": 4,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 5}},
             "layers": [dict(kinds[i % 2], mlp=mlp) for i in range(layers)]}
 
 
