@@ -95,7 +95,7 @@ def time_prefill(engine, runs: int = 5, n_tokens: int = PROMPT_LEN, warmups: int
 
 
 def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, profile: bool = False,
-                prompt_len: int = PROMPT_LEN):
+                prompt_len: int = PROMPT_LEN, most: int = 8):
     """Median seconds for exactly `steps` decode steps of `batch` requests that each hold a
     `prompt_len`-token prompt (greedy sampling on the device), the requests' lengths at the middle of that
     run, and, with `profile`, the kernels of one more run by their share of its device time."""
@@ -120,7 +120,7 @@ def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, p
         loop.run(steps)
         torch.cuda.synchronize()
         samples.append((time.perf_counter() - t0, lens))
-    top = kernel_shares(lambda: loop.run(min(steps, 16))) if profile else None
+    top = kernel_shares(lambda: loop.run(min(steps, 16)), most=most) if profile else None
     for rid in rids:
         engine.release(rid)
     dt, seq_lens = sorted(samples, key=lambda s: s[0])[len(samples) // 2]
@@ -384,9 +384,9 @@ def compare_designs(args) -> int:
             row["prefill_frac_of_peak"] = round(R.prefill_flops(engine, args.prefill_tokens) / prefill_s / R.PEAK_FLOPS[args.dtype], 4)
             if profile:
                 ids = seeded_prompt(5, args.prefill_tokens, vocab)
-                row["prefill_kernels"] = kernel_shares(lambda: (engine.step([("k", ids, [len(ids) - 1])]), engine.release("k")), most=10)
+                row["prefill_kernels"] = kernel_shares(lambda: (engine.step([("k", ids, [len(ids) - 1])]), engine.release("k")), most=14)
             print(f"[bench] {design} width {width}: decode", file=sys.stderr, flush=True)
-            dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=profile, prompt_len=args.prompt_len)
+            dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=profile, prompt_len=args.prompt_len, most=14)
             row["decode_tok_s"] = round(args.batch * args.steps / dt, 1)
             row["decode_ms_per_step"] = round(dt / args.steps * 1e3, 4)
             row["decode_frac_of_hbm"] = round(R.decode_bytes(engine, seq_lens) / (dt / args.steps) / R.HBM_BYTES_PER_S, 4)
